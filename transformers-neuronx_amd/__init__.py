@@ -1,4 +1,4 @@
-"""An inference engine for decoder-only language models (OPT, Ratesun, Sunatar) on one AMD MI355X."""
+"""An inference engine for decoder-only language models (OPT, Ratesun, Sunatar, Tadolix) on one AMD MI355X."""
 __version__ = "0.1.0"
 
 from .config import ContinuousBatchingConfig, EngineConfig, GenerationConfig, NeuronConfig  # noqa: F401
@@ -16,6 +16,9 @@ def __getattr__(name):
     if name == "SunatarForSampling":
         from .sunatar import model
         return model.SunatarForSampling
+    if name == "TadolixForSampling":
+        from .tadolix import model
+        return model.TadolixForSampling
     if name == "NeuronAutoModelForCausalLM":
         from .modeling_auto import NeuronAutoModelForCausalLM
         return NeuronAutoModelForCausalLM

@@ -107,6 +107,9 @@ class CacheManager:
                         count = int(np.prod(dims))
                         whole = torch.empty(g.pool.num_pages, count + page_pad_bytes // item, dtype=dtype, device=device)
                         lc.pages[name] = whole[:, :count].view(g.pool.num_pages, *dims)
+                    sdt = getattr(torch, need.state_dtype)
+                    for name, shape in need.state_shapes:       # a mixer that keeps pages and a fixed state
+                        lc.state[name] = torch.zeros(max_seqs, *shape, dtype=sdt, device=device)
                 self.caches[cid] = lc
             elif need.kind == "state":
                 lc = LayerCache(cid, None)

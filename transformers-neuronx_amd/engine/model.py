@@ -179,6 +179,9 @@ class DecoderModel:
             ctx.call_state = caches[state_id] if state_id is not None else None
             stream = self.layers[layer].block.forward(stream, ctx, cache)
             debug.tap(f"call{call}.layer{layer}", stream.x)
+        if stream.copies is not None and (stream.x is None or stream.pending is not None):
+            # an arrangement that keeps several copies of the stream: their sum is what the head reads
+            stream = Stream(self.ops.hyper_sum(stream.copies, stream.pending))
         return debug.tap("logits", self.head.forward(stream, ctx))
 
 

@@ -59,6 +59,36 @@ class ReferenceOps:
         x = src.float() * scale
         return x, (x.to(dtype) if want_compute else None)
 
+    def add_sinusoid(self, src, positions, freqs, dtype, want_compute, scale=1.0):
+        """float32 `src * scale` plus, at elements 2i and 2i + 1, the sine and the cosine of position * freqs[i]
+        (the angle a float32 product)."""
+        angle = positions.float()[:, None] * freqs.float()[None, :]
+        x = src.float() * scale + torch.stack([torch.sin(angle), torch.cos(angle)], dim=-1).reshape(src.shape)
+        return x, (x.to(dtype) if want_compute else None)
+
+    # ---------------------------------------------------------------- several copies of the stream
+
+    @staticmethod
+    def _join(copies, pending):
+        """`copies[b] <- sum_a mix[a, b] copies[a] + out[b] y` for pending = (y, mix, out), in place."""
+        if pending is not None:
+            y, mix, out = pending
+            copies.copy_(torch.einsum("ab,atd->btd", mix.float(), copies) + out.float()[:, None, None] * y.float()[None])
+
+    def hyper_step(self, copies, pending, read, norm_weight, eps, dtype, want_f32, want_compute):
+        """Joins what is pending to the float32 copies `[s, T, width]` (in place), then
+        h = u / sqrt(mean(u^2) + eps) * norm_weight with u = sum_a read[a] copies[a]; returns (h in float32 or None,
+        h in `dtype` or None)."""
+        self._join(copies, pending)
+        u = torch.einsum("a,atd->td", read.float(), copies)
+        h = u * torch.rsqrt((u * u).mean(-1, keepdim=True) + eps) * norm_weight.float()
+        return (h if want_f32 else None), (h.to(dtype) if want_compute else None)
+
+    def hyper_sum(self, copies, pending):
+        """Joins what is pending (in place) and returns the float32 sum of the copies."""
+        self._join(copies, pending)
+        return copies.sum(0)
+
     # ---------------------------------------------------------------- norms
 
     def layernorm(self, x, weight, bias, eps, dtype, want_f32, want_compute, center=True):
@@ -395,7 +425,7 @@ class ReferenceOps:
     # ---------------------------------------------------------------- normed, turned and blended projections
 
     def qkv_prepare(self, proj, num_heads, num_kv, head_size, value_size, cache_head, q_weight, k_weight, eps, freqs,
-                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages):
+                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages, per_head=False):
         """From the float32 projections `proj` `[T, H n + G n + G v]` (bias added) to the queries and the cache:
         the queries and the keys are each scaled to unit root mean square over their whole width and weighted
         (`q_weight`, `k_weight`; None: not), the first `2 len(freqs)` elements of every head are turned by
@@ -408,7 +438,14 @@ class ReferenceOps:
         nq, nk, nv = num_heads * head_size, num_kv * head_size, num_kv * value_size
         x = proj.float()
         q, k, v = x[:, :nq], x[:, nq:nq + nk], x[:, nq + nk:nq + nk + nv]
-        if q_weight is not None:
+        if per_head:
+            # every head to unit root mean square by itself; the weights, if any, are still one a projection element
+            q, k = q.reshape(t, num_heads, head_size), k.reshape(t, num_kv, head_size)
+            q = (q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps)).reshape(t, nq)
+            k = (k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps)).reshape(t, nk)
+            if q_weight is not None:
+                q, k = q * q_weight.float(), k * k_weight.float()
+        elif q_weight is not None:
             q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * q_weight.float()
             k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * k_weight.float()
         q, k = q.reshape(t, num_heads, head_size), k.reshape(t, num_kv, head_size)
@@ -441,6 +478,147 @@ class ReferenceOps:
         out = torch.zeros(t, num_heads, cache_head, dtype=self.dtype, device=proj.device)
         out[:, :, :head_size] = (q * scale).to(self.dtype)
         return out.reshape(t, num_heads * cache_head)
+
+    def attention_scored(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None,
+                         chunk=None, softcap=None, distance_bias=None, gate=None, value_size=None, out=None,
+                         out_scale=1.0):
+        """Attention whose scores or mask are not the plain ones. For a query at position i and a key at j <= i of
+        its request: s = q . k (the query comes scaled); with `softcap` c, s <- c tanh(s / c); with
+        `distance_bias` (float32 `[heads, D + 1]`), s <- s + distance_bias[head, min(i - j, D)]. Visible are the
+        keys with i - j < window (if given) and floor(j / chunk) = floor(i / chunk) (if given). Softmax over the
+        visible keys, times the values. `gate` (float32 `[T, heads * value_size]`, rows may lie apart): the first
+        `value_size` elements of every head are multiplied by sigmoid(gate). The result times `out_scale` goes to
+        `out` (`[T, heads * head_size]` in the compute dtype, rows may lie apart) or to a new tensor."""
+        t = q.shape[0]
+        value_size = head_size if value_size is None else value_size
+        res = torch.empty(t, num_heads, head_size, dtype=torch.float32, device=q.device)
+        ps = view.page_size
+        group = num_heads // num_kv_heads
+        starts = ctx.run_start.tolist()
+        for r in range(ctx.num_requests):
+            s, e = starts[r], starts[r + 1]
+            if e == s:
+                continue
+            total = int(ctx.cached_lens_host[r]) + (e - s)
+            nb = -(-total // ps)
+            pages = view.block_table[r, :nb].long().clamp(min=0)
+            keys = k_pages[pages].float().permute(1, 0, 2, 3).reshape(num_kv_heads, nb * ps, head_size)[:, :total]
+            vals = v_pages[pages].float().permute(1, 2, 0, 3).reshape(num_kv_heads, head_size, nb * ps)[:, :, :total]
+            vals = torch.where(torch.isfinite(vals), vals, torch.zeros_like(vals))
+            keys = torch.where(torch.isfinite(keys), keys, torch.zeros_like(keys))
+            qr = q[s:e].float().reshape(e - s, num_heads, head_size).permute(1, 0, 2)
+            keys = keys.repeat_interleave(group, dim=0)
+            vals = vals.repeat_interleave(group, dim=0)
+            scores = qr @ keys.transpose(1, 2)                       # [heads, run, total]
+            if softcap:
+                scores = softcap * torch.tanh(scores / softcap)
+            pos = ctx.positions[s:e].long().unsqueeze(1)
+            j = torch.arange(total, device=q.device).unsqueeze(0)
+            allowed = j <= pos
+            if distance_bias is not None:
+                far = distance_bias.shape[1] - 1
+                scores = scores + distance_bias.float()[:, (pos - j).clamp(0, far)]
+            if window is not None:
+                allowed &= j > pos - window
+            if chunk is not None:
+                allowed &= (j // chunk) == (pos // chunk)
+            scores = scores.masked_fill(~allowed.unsqueeze(0), float("-inf"))
+            p = torch.softmax(scores, dim=-1)
+            res[s:e] = (p @ vals.transpose(1, 2)).permute(1, 0, 2)
+        if gate is not None:
+            res[:, :, :value_size] *= torch.sigmoid(gate.float()).reshape(t, num_heads, value_size)
+        res = (res * out_scale).reshape(t, num_heads * head_size)
+        if out is None:
+            return res.to(self.dtype)
+        out.copy_(res)
+        return out
+
+    # ---------------------------------------------------------------- recurrences
+
+    def min_gru(self, proj, inner, ctx, carried, out=None, out_scale=1.0):
+        """The minimal gated recurrence over a step's runs. `proj` float32 `[T, 3 inner]` = [z' | u | g] (biases
+        added): z = sigmoid(z'), c = u + 1/2 where u >= 0 and sigmoid(u) below, S <- (1 - z) S + z c; the result
+        is S silu(g) times `out_scale`, `[T, inner]` in the compute dtype (into `out`, whose rows may lie apart).
+        `carried` float32 `[slots, 2, inner]`: the token at position p reads place (p - 1) & 1 (zeros at p = 0) and
+        writes place p & 1."""
+        x = proj.float()
+        z, u, g = torch.sigmoid(x[:, :inner]), x[:, inner:2 * inner], x[:, 2 * inner:3 * inner]
+        cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+        res = torch.empty(x.shape[0], inner, dtype=torch.float32, device=x.device)
+        start = 0
+        for r in range(ctx.num_requests):
+            n, slot, have = int(ctx.run_lens_host[r]), int(ctx.slots_host[r]), int(ctx.cached_lens_host[r])
+            s = carried[slot, (have - 1) & 1].clone() if have > 0 else torch.zeros_like(carried[slot, 0])
+            for i in range(start, start + n):
+                s = (1.0 - z[i]) * s + z[i] * cand[i]
+                res[i] = s
+            if n:
+                carried[slot, (have + n - 1) & 1] = s
+            start += n
+        res = res * (g * torch.sigmoid(g)) * out_scale
+        if out is None:
+            return res.to(self.dtype)
+        out.copy_(res)
+        return out
+
+    def channel_conv(self, x, weight, bias, ctx, state):
+        """A causal convolution over the request's tokens on every channel, with a bias:
+        u_t = bias + sum_j weight[:, j] x_(t - taps + 1 + j), zeros before the request's start. `x` float32
+        `[T, channels]` (rows may lie apart), `weight` `[channels, taps]`. `state` float32 `[slots, taps, channels]`
+        holds the input at position p at place p mod taps and takes the run's last ones. Returns (u in float32, u
+        in the compute dtype)."""
+        taps = weight.shape[1]
+        x = x.float()
+        out = torch.empty_like(x)
+        start = 0
+        for r in range(ctx.num_requests):
+            n, slot, have = int(ctx.run_lens_host[r]), int(ctx.slots_host[r]), int(ctx.cached_lens_host[r])
+            run = x[start:start + n]
+            if taps > 1:
+                before = [state[slot, p % taps].float() if p >= 0 else torch.zeros_like(run[0])
+                          for p in range(have - (taps - 1), have)]
+                seq = torch.cat([torch.stack(before), run], dim=0)
+                for i in range(max(0, n - (taps - 1)), n):
+                    state[slot, (have + i) % taps] = run[i]
+            else:
+                seq = run
+            acc = bias.float()[None, :].expand(n, -1).clone()
+            for j in range(taps):
+                acc = acc + weight[:, j].float()[None, :] * seq[j:j + n]
+            out[start:start + n] = acc
+            start += n
+        return out, out.to(self.dtype)
+
+    def gated_linear_recurrence(self, gates, gate_bias, u, y, rate, ctx, carried, out=None, out_scale=1.0):
+        """The real-gated linear recurrence over a step's runs. `gates` float32 `[T, blocks, 2 w]`: a part's
+        pre-activations of the recurrence gate (the first w) and of the input gate, `gate_bias` `[blocks, 2 w]`
+        their biases; `u` float32 `[T, blocks w]`; `y` float32 `[T, blocks w]` (rows may lie apart), through
+        gelu_tanh here; `rate` `[blocks w]` = -8 softplus(lam).
+        a = exp(rate sigmoid(r')), S <- a S + sqrt(1 - a^2) sigmoid(i') u; the result S gelu_tanh(y) times
+        `out_scale` in the compute dtype. `carried` as in `min_gru`."""
+        t, blocks, two_w = gates.shape
+        w = two_w // 2
+        pre = gates.float() + gate_bias.float()[None]
+        r = torch.sigmoid(pre[:, :, :w]).reshape(t, blocks * w)
+        i = torch.sigmoid(pre[:, :, w:]).reshape(t, blocks * w)
+        a = torch.exp(rate.float()[None, :] * r)
+        inp = torch.sqrt(1.0 - a * a) * i * u.float()
+        res = torch.empty(t, blocks * w, dtype=torch.float32, device=u.device)
+        start = 0
+        for q in range(ctx.num_requests):
+            n, slot, have = int(ctx.run_lens_host[q]), int(ctx.slots_host[q]), int(ctx.cached_lens_host[q])
+            s = carried[slot, (have - 1) & 1].clone() if have > 0 else torch.zeros_like(carried[slot, 0])
+            for k in range(start, start + n):
+                s = a[k] * s + inp[k]
+                res[k] = s
+            if n:
+                carried[slot, (have + n - 1) & 1] = s
+            start += n
+        res = res * self.activation(y.float(), "gelu_new") * out_scale
+        if out is None:
+            return res.to(self.dtype)
+        out.copy_(res)
+        return out
 
     # ---------------------------------------------------------------- the matrix memory
 

@@ -3,4 +3,4 @@ from .base import (BLOCKS, EMBEDDINGS, FEED_FORWARDS, HEADS, MIXERS, NORMS, POSI
                    register_embedding, register_feed_forward, register_head, register_mixer,
                    register_norm, register_position)
 from .spec import LayerCall, LayerSpec, ModelSpec, ParamDecl, PartSpec
-from . import block, embedding, feed_forward, mixer, norm, position  # noqa: F401  (register the built-in parts)
+from . import block, embedding, feed_forward, mixer, norm, position, recurrent  # noqa: F401  (register the built-in parts)

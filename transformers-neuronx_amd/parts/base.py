@@ -23,7 +23,8 @@ class CacheNeed:
          `(kv_heads, head_size, "page")`. `window` (tokens) lets pages be given back once every later
          query is past them, None keeps them all.
     kind 'state': fixed size per request. `state_shapes` is ((name, dims), ...); a slot is zeroed when a
-         request gets it.
+         request gets it. A 'paged' need may name `state_shapes` too (a mixer that keeps both: pages that grow
+         and a state of fixed size).
     """
     kind: str
     kv_heads: int = 0
@@ -199,11 +200,16 @@ class Stream:
     """The residual stream between layers: float32 `[T, hidden]`, and beside it a
     copy in the compute dtype when the last part that wrote it made one. `history`, for arrangements that
     read what earlier layers left: float32 `[slots, T, hidden]` with `filled` slots written (slot 0 the
-    embedded tokens, slot i + 1 the result of the i-th call), or None."""
+    embedded tokens, slot i + 1 the result of the i-th call), or None. `copies`, for arrangements that keep
+    several copies of the stream: float32 `[copies, T, hidden]`; `x` is then None until the copies are summed,
+    and `pending` = (y, mix, out) is a sublayer's result that has not joined the copies yet (whoever reads
+    the copies next applies it in the same launch)."""
     x: "object"
     compute: Optional["object"] = None
     history: Optional["object"] = None
     filled: int = 0
+    copies: Optional["object"] = None
+    pending: Optional[tuple] = None
 
 
 class _Registry:

@@ -206,3 +206,111 @@ class SandwichBlock(Block):
             raise ValueError(f"this call averages {self.depth_average} results and {filled + 1} are there")
         debug.tap("own_result", x)
         return Stream(ops.weighted_sum(history, self.depth_w, filled + 1), None, history, filled + 1)
+
+
+@register_block("hyper")
+class HyperConnectionBlock(Block):
+    """Pre-norm sublayers around several copies of the residual stream (hyper-connections). The copies x_1 .. x_s
+    all start as the embedded tokens. For a sublayer f (the mixer, then the feed-forward, where the layer has one)
+    with its own weights `in` [s], `out` [s] and `mix` [s, s] (indexed [from, to]):
+
+        u = sum_a in[a] x_a,   y = f(norm(u)),   x_b <- sum_a mix[a, b] x_a + out[b] y     (all b at once, from the old copies)
+
+    `streams=0` is the plain residual sum x <- x + f(norm(x)): one copy and no weights. With `taps`, what the mixer
+    reads is first replaced by h + conv(h), a causal convolution over the request's tokens on every channel
+    (weights `[width, taps]`, zeros before the request's start); its last taps - 1 inputs are per-request state.
+    The copies, the norms, the sums and the state are float32. When the last call of the run order is through,
+    the model sums the copies.
+
+    A sublayer's result does not join the copies at once: it is left `pending` on the stream, and whoever reads
+    the copies next (the next sublayer's weighted sum and norm, or the sum at the end) applies it in the same
+    launch."""
+
+    recordable = True
+
+    def __init__(self, mixer, feed_forward, mixer_norm, feed_forward_norm, *, streams: int, taps: int = 0,
+                 conv_name: str = "conv", names=("hc1.", "hc2."), parts=("in", "out", "mix")):
+        """`names`: the prefixes of the mixer's and the feed-forward's stream weights, relative to the layer's;
+        `parts`: what the three tensors are called under them."""
+        super().__init__(mixer, feed_forward, mixer_norm, feed_forward_norm)
+        self.streams, self.taps, self.conv_name = int(streams), int(taps), conv_name
+        self.names, self.part_names = tuple(names), tuple(parts)
+        self.has_ff = not getattr(feed_forward, "absent", False)
+        self.width = mixer_norm.width
+        if self.streams < 0 or self.taps < 0:
+            raise ValueError(f"hyper-connections with {streams} streams and {taps} taps")
+        for norm in (mixer_norm,) + ((feed_forward_norm,) if self.has_ff else ()):
+            if not hasattr(norm, "fused_form") or norm.fused_form()[2]:
+                raise ValueError("the norm behind the weighted sum of the copies is one that only scales (rms_norm)")
+
+    def state_need(self):
+        if self.taps > 1:
+            from .base import CacheNeed
+            return CacheNeed("state", state_shapes=(("inputs", (1, self.taps, self.width)),))
+        return None
+
+    def _sublayers(self):
+        return self.names[:2 if self.has_ff else 1]
+
+    def param_decls(self, prefix: str):
+        from .spec import ParamDecl
+        d = []
+        s = self.streams
+        if s:
+            i, o, m = self.part_names
+            for name in self._sublayers():
+                d += [ParamDecl(prefix + name + i, (s,), "vector", "around_mean"),
+                      ParamDecl(prefix + name + o, (s,), "vector", "around_one"),
+                      ParamDecl(prefix + name + m, (s, s), "vector", "around_mean")]
+        if self.taps > 0:
+            d.append(ParamDecl(prefix + self.conv_name, (self.width, self.taps), "vector"))
+        return d
+
+    def load(self, tensors, prefix, ops, dtype) -> None:
+        import torch
+        super().load(tensors, prefix, ops, dtype)
+        self.weights = []
+        for name in self._sublayers():
+            if self.streams:
+                i, o, m = (tensors[prefix + name + p].float().contiguous() for p in self.part_names)
+            else:
+                one = torch.ones(1, dtype=torch.float32, device=getattr(ops, "device", "cpu"))
+                i, o, m = one, one, one.view(1, 1)
+            self.weights.append((i, o, m))
+        self.conv_w = tensors[prefix + self.conv_name] if self.taps > 0 else None
+
+    def _read(self, stream: Stream, which: int, norm, want_f32: bool):
+        """The copies with what is pending joined, and norm(sum_a in[a] x_a) in float32 or in the compute dtype."""
+        weight, _, _, eps = norm.fused_form()
+        h32, hc = self.ops.hyper_step(stream.copies, stream.pending, self.weights[which][0], weight, eps, self.dtype,
+                                      want_f32, not want_f32)
+        return h32 if want_f32 else hc
+
+    def forward(self, stream: Stream, ctx, cache) -> Stream:
+        ops = self.ops
+        copies = stream.copies
+        if copies is None:          # the first call of the run order: every copy is the embedded tokens
+            copies = stream.x.unsqueeze(0).repeat(max(1, self.streams), 1, 1)
+            stream = Stream(None, None, copies=copies)
+        elif copies.shape[0] != max(1, self.streams):
+            raise ValueError(f"the stream has {copies.shape[0]} copies, this layer {max(1, self.streams)}")
+        if self.taps > 0:
+            h = self._read(stream, 0, self.mixer_norm, True)
+            state = ctx.call_state.state["inputs"] if self.taps > 1 else None
+            h = ops.input_conv(h, self.conv_w, state, 0, ctx, self.dtype)
+        else:
+            h = self._read(stream, 0, self.mixer_norm, False)
+        y = self.mixer.forward(h, ctx, cache, None)
+        stream = Stream(None, None, copies=copies, pending=(y, self.weights[0][2], self.weights[0][1]))
+        if debug.tapping():
+            debug.tap("after_mixer", ops.hyper_sum(copies, stream.pending))
+            stream.pending = None
+        if self.has_ff:
+            h = self._read(stream, 1, self.feed_forward_norm, False)
+            y = self.feed_forward.forward(h, ctx, None)
+            stream = Stream(None, None, copies=copies, pending=(y, self.weights[1][2], self.weights[1][1]))
+        if debug.tapping():
+            # what a tap of the stream after this call sees: the sum of the copies
+            stream.x = ops.hyper_sum(copies, stream.pending)
+            stream.pending = None
+        return stream

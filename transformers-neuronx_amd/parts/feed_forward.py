@@ -57,6 +57,40 @@ class DenseFeedForward(FeedForward):
         return self.ops.linear(inner, self.w2, self.b2, residual=residual, out_f32=True, f32_by_library=residual is None)
 
 
+@register_feed_forward("gated")
+class GatedFeedForward(FeedForward):
+    """`W_down (act(W_gate h) * (W_up h))`, no biases: gate and up rows are one product, the activation and the
+    product of the two halves are made on its float32 sums and rounded once."""
+
+    recordable = True
+
+    def __init__(self, width: int, inner: int, activation: str, names, weight_suffix: str = ""):
+        """`names`: the checkpoint's names of the gate, up and down matrices; `activation`: "gelu_new" (the tanh
+        form) or "silu"."""
+        if activation not in ("gelu_new", "silu"):
+            raise ValueError(f"a gated feed-forward's activation is gelu_new or silu, got {activation!r}")
+        self.width, self.inner, self.activation = width, inner, activation
+        self.names, self.weight_suffix = tuple(names), weight_suffix
+
+    def param_decls(self, prefix: str) -> List[ParamDecl]:
+        g, u, d = (f"{prefix}{n}{self.weight_suffix}" for n in self.names)
+        return [ParamDecl(g, (self.inner, self.width)), ParamDecl(u, (self.inner, self.width)),
+                ParamDecl(d, (self.width, self.inner))]
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        import torch
+        super().load(tensors, prefix, ops, dtype)
+        g, u, d = (f"{prefix}{n}{self.weight_suffix}" for n in self.names)
+        self.w_in = ops.prepare_weight(torch.cat([tensors[g], tensors[u]], dim=0).contiguous())
+        self.w_down = ops.prepare_weight(tensors[d])
+
+    def forward(self, h, ctx, residual):
+        inner = self.ops.gated_activation(self.ops.linear(h, self.w_in, None, out_f32=True, f32_by_library=True),
+                                          self.activation)
+        return self.ops.linear(inner, self.w_down, None, residual=residual, out_f32=True,
+                               f32_by_library=residual is None)
+
+
 @register_feed_forward("none")
 class NoFeedForward(FeedForward):
     """A layer without a feed-forward: the stream passes."""

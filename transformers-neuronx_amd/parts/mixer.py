@@ -8,6 +8,28 @@ from .base import POSITIONS, CacheNeed, Mixer, register_mixer
 from .spec import ParamDecl
 
 
+def distance_bucket(n: int, rows: int, max_distance: int) -> int:
+    """The row of a distance-bias table for the distance n >= 0 between a query and a key: the distance itself
+    below rows / 2, then logarithmic steps that reach the last row at `max_distance`."""
+    half = rows // 2
+    if n < half:
+        return n
+    return min(rows - 1, half + int(math.floor(math.log(n / half) / math.log(max_distance / half) * (rows - half))))
+
+
+def bias_by_distance(table: torch.Tensor, max_distance: int) -> torch.Tensor:
+    """float32 `[heads, max_distance + 1]` from a table `[rows, heads]`: what a head adds to the score of a key n
+    tokens back, at column min(n, max_distance) (every distance from `max_distance` on falls into the last row).
+    The buckets are worked out once, on the host, in double precision."""
+    rows = table.shape[0]
+    if rows < 2 or max_distance <= rows // 2:
+        raise ValueError(f"a distance bias of {rows} rows up to distance {max_distance}: the rows beyond the first "
+                         f"half need a distance beyond {rows // 2} to spread over")
+    rows_of = torch.tensor([distance_bucket(n, rows, max_distance) for n in range(max_distance)] + [rows - 1],
+                           dtype=torch.long, device=table.device)
+    return table.float()[rows_of].t().contiguous()
+
+
 @register_mixer("attention")
 class Attention(Mixer):
     """Softmax attention over a paged key/value cache.
@@ -33,7 +55,9 @@ class Attention(Mixer):
     def __init__(self, width: int, num_heads: int, head_size: int, names, num_kv_heads: Optional[int] = None,
                  bias: bool = True, window: Optional[int] = None, scale: Optional[float] = None,
                  own_kv: bool = True, rotation=None, value_size: Optional[int] = None, out_bias: Optional[bool] = None,
-                 qk_norm=None, value_mix=None, weight_suffix: str = ".weight", bias_suffix: str = ".bias"):
+                 qk_norm=None, value_mix=None, weight_suffix: str = ".weight", bias_suffix: str = ".bias",
+                 softcap: Optional[float] = None, distance_bias=None, chunk: Optional[int] = None,
+                 out_gate: Optional[str] = None):
         """`names`: the checkpoint's names of the query, key, value and output projections, relative to
         the mixer's prefix (the architecture's spec gives them); a matrix's name adds `weight_suffix`, a bias's
         `bias_suffix`. `out_bias`: whether the output projection has a bias (as the others, if not said).
@@ -46,9 +70,22 @@ class Attention(Mixer):
         v = (1 - l) v + l v_first with l the scalar tensor `name`; the blended values are what is cached. The
         first blends nothing and has no such tensor. A rotation whose pairs are not neighbours
         (`interleaved=False`) hands its frequencies to the kernel that norms, turns and stores.
+        With `per_head` in `qk_norm` every head is scaled to unit root mean square by itself, and with
+        `weighted=False` there are no weight tensors.
         These take the float32 route: the projection's float32 result goes through one kernel (`ops.qkv_prepare`)
         that norms, turns, scales, blends and stores, and heads of unequal sizes are cached filled up with
-        zeros to one size, a multiple of 16."""
+        zeros to one size, a multiple of 16.
+
+        What changes the scores or the mask (the route above, and `ops.attention_scored` in the place of
+        `ops.attention`): `softcap` c: a score s becomes c tanh(s / c) (after the scale). `distance_bias` =
+        {name, max_distance, rows}: the tensor `name` `[rows, heads]` holds a bias a head for every bucket of the
+        distance n = i - j between query and key, added after the cap: bucket(n) = n below rows / 2, and from
+        there on logarithmic steps up to `max_distance`, min(rows - 1, rows/2 + floor(ln(n / (rows/2)) /
+        ln(max_distance / (rows/2)) * (rows - rows/2))); `rows` None: the checkpoint's tensor says. `chunk` m: a
+        query at position i sees the keys j <= i with floor(j / m) = floor(i / m), positions counted from the
+        request's start. `out_gate`: the name of a matrix W_g `[heads * value_size, width]`; the heads' results
+        side by side are multiplied by sigmoid(W_g h) before the output projection (the gate's rows ride in the
+        one input projection)."""
         self.width, self.num_heads, self.head_size = width, num_heads, head_size
         self.num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
         if self.num_heads % self.num_kv_heads:
@@ -58,7 +95,15 @@ class Attention(Mixer):
         self.value_mix = dict(value_mix) if value_mix else None
         self.rotation = POSITIONS.build(rotation) if rotation is not None else None
         halves = self.rotation is not None and not getattr(self.rotation, "interleaved", True)
-        self.prepared = bool(self.qk_norm or self.value_mix or halves or self.value_size != head_size)
+        self.softcap = float(softcap) if softcap else None
+        self.distance_bias = dict(distance_bias) if distance_bias else None
+        self.chunk = int(chunk) if chunk else None
+        self.out_gate = out_gate
+        if self.chunk is not None and window is not None:
+            raise ValueError("an attention mixer masks by a window or by chunks, not both")
+        self.scored = bool(self.softcap or self.distance_bias or self.chunk or out_gate)
+        self.prepared = bool(self.qk_norm or self.value_mix or halves or self.value_size != head_size or self.scored)
+        self.defer_out = False      # set by a mixer that runs this one beside another and owns the output product
         if self.prepared:
             if not own_kv:
                 raise ValueError("a mixer that norms, blends or fills up its heads makes its own keys and values")
@@ -97,9 +142,14 @@ class Attention(Mixer):
         d.append(ParamDecl(f"{prefix}{on}{ws}", (self.width, self.num_heads * self.value_size)))
         if self.has_out_bias:
             d.append(ParamDecl(f"{prefix}{on}{bs}", (self.width,), "vector"))
-        if self.qk_norm:
+        if self.qk_norm and self.qk_norm.get("weighted", True):
             d += [ParamDecl(f"{prefix}{qn}{self.qk_norm['suffix']}", (q_out,), "vector", "around_one"),
                   ParamDecl(f"{prefix}{kn}{self.qk_norm['suffix']}", (kv_out,), "vector", "around_one")]
+        if self.distance_bias:
+            d.append(ParamDecl(f"{prefix}{self.distance_bias['name']}", (self.distance_bias.get("rows"), self.num_heads),
+                               "vector"))
+        if self.out_gate:
+            d.append(ParamDecl(f"{prefix}{self.out_gate}{ws}", (self.num_heads * self.value_size, self.width)))
         if self.value_mix and not self.value_mix["first"]:
             d.append(ParamDecl(f"{prefix}{self.value_mix['name']}", (), "vector", "around_half"))
         if self.rotation is not None:
@@ -110,7 +160,7 @@ class Attention(Mixer):
         super().load(tensors, prefix, ops, dtype)
         qn, kn, vn, on = self.names
         ws, bs = self.weight_suffix, self.bias_suffix
-        ins = [qn] + ([kn, vn] if self.own_kv else [])
+        ins = [qn] + ([kn, vn] if self.own_kv else []) + ([self.out_gate] if self.out_gate else [])
         # One fused projection: a plain concatenation of the rows (the reference's
         # fused form interleaves per tensor-parallel shard, utils.py:189-242).
         self.w_qkv = ops.prepare_weight(torch.cat([tensors[f"{prefix}{n}{ws}"] for n in ins], dim=0).contiguous())
@@ -122,8 +172,15 @@ class Attention(Mixer):
             wide = w_out.new_zeros(self.width, self.num_heads, self.cache_head)
             wide[:, :, :self.value_size] = w_out.view(self.width, self.num_heads, self.value_size)
             w_out = wide.view(self.width, self.num_heads * self.cache_head).contiguous()
-        self.w_out = ops.prepare_weight(w_out)
+        if self.defer_out:
+            self.w_out_raw, self.w_out = w_out, None
+        else:
+            self.w_out = ops.prepare_weight(w_out)
         self.b_out = tensors[f"{prefix}{on}{bs}"] if self.has_out_bias else None
+        self.bias_by_distance = None
+        if self.distance_bias:
+            self.bias_by_distance = bias_by_distance(tensors[f"{prefix}{self.distance_bias['name']}"],
+                                                     int(self.distance_bias["max_distance"]))
         self.turn = None
         self.q_norm = self.k_norm = self.mix_weight = self.freqs = None
         if self.rotation is not None:
@@ -132,7 +189,7 @@ class Attention(Mixer):
                 self.freqs = self.rotation.frequencies()
             else:
                 self.turn = self.rotation.pair_tables(self.head_size)     # the pairwise form: applied by the projection
-        if self.qk_norm:
+        if self.qk_norm and self.qk_norm.get("weighted", True):
             self.q_norm = tensors[f"{prefix}{qn}{self.qk_norm['suffix']}"]
             self.k_norm = tensors[f"{prefix}{kn}{self.qk_norm['suffix']}"]
         if self.value_mix and not self.value_mix["first"]:
@@ -151,12 +208,34 @@ class Attention(Mixer):
 
     def flops_per_token(self, keys: float = 0.0) -> float:
         seen = min(keys, self.window) if self.window else keys
+        if self.chunk:
+            seen = min(keys, (self.chunk + 1) / 2.0)      # a query sees half a chunk on average
         # q k^T and p v
         return super().flops_per_token(keys) + 2.0 * self.num_heads * (self.head_size + self.value_size) * seen
+
+    # ---- beside another mixer (`side_by_side`): the heads' results go into a slice of a buffer that the two
+    # share, and the mixer that runs them owns the one output product
+
+    def inner_width(self) -> int:
+        return self.num_heads * self.cache_head
+
+    def out_matrix(self):
+        w, self.w_out_raw = self.w_out_raw, None
+        return w
+
+    def inner_into(self, h, ctx, cache, out, scale: float) -> None:
+        if not self.prepared or self.has_out_bias:
+            raise ValueError("an attention mixer beside another takes the float32 route and has no output bias")
+        self._inner_prepared(h, ctx, cache, ctx.groups[cache.group], out, scale)
 
     def _forward_prepared(self, h, ctx, cache, residual, view):
         """The float32 route: projection with its bias, one kernel that norms, turns, scales, blends and stores,
         attention over heads of the cache's size, the output projection."""
+        ops = self.ops
+        c = self._inner_prepared(h, ctx, cache, view, None, 1.0)
+        return ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
+
+    def _inner_prepared(self, h, ctx, cache, view, out, out_scale):
         ops = self.ops
         proj = ops.linear(h, self.w_qkv, self.b_qkv, out_f32=True, f32_by_library=True)
         first = None
@@ -164,7 +243,8 @@ class Attention(Mixer):
             key = ("value mix", self.value_mix["key"])
             if self.value_mix["first"]:
                 # what the later layers blend with: this step's values as this layer made them
-                ctx.memo[key] = proj[:, (self.num_heads + self.num_kv_heads) * self.head_size:]
+                at = (self.num_heads + self.num_kv_heads) * self.head_size
+                ctx.memo[key] = proj[:, at:at + self.num_kv_heads * self.value_size]
             else:
                 first = ctx.memo.get(key)
                 if first is None:
@@ -173,10 +253,19 @@ class Attention(Mixer):
         q = ops.qkv_prepare(proj, self.num_heads, self.num_kv_heads, self.head_size, self.value_size, self.cache_head,
                             self.q_norm, self.k_norm, self.qk_norm["eps"] if self.qk_norm else 0.0, self.freqs,
                             bool(rot.interleaved) if rot is not None else False, self.scale, self.mix_weight, first,
-                            ctx, view, cache.k_pages, cache.v_pages)
-        c = ops.attention(q, self.num_heads, self.num_kv_heads, self.cache_head, ctx, view, cache.k_pages,
-                          cache.v_pages, self.window)
-        return ops.linear(c, self.w_out, self.b_out, residual=residual, out_f32=True)
+                            ctx, view, cache.k_pages, cache.v_pages,
+                            **({"per_head": True} if (self.qk_norm or {}).get("per_head") else {}))
+        if not self.scored and out is None:
+            return ops.attention(q, self.num_heads, self.num_kv_heads, self.cache_head, ctx, view, cache.k_pages,
+                                 cache.v_pages, self.window)
+        gate = None
+        if self.out_gate:
+            at = self.num_heads * self.head_size + self.num_kv_heads * (self.head_size + self.value_size)
+            gate = proj[:, at:at + self.num_heads * self.value_size]
+        return ops.attention_scored(q, self.num_heads, self.num_kv_heads, self.cache_head, ctx, view, cache.k_pages,
+                                    cache.v_pages, window=self.window, chunk=self.chunk, softcap=self.softcap,
+                                    distance_bias=self.bias_by_distance, gate=gate, value_size=self.value_size,
+                                    out=out, out_scale=out_scale)
 
     def forward(self, h, ctx, cache, residual):
         if cache.writes != self.own_kv:

@@ -56,20 +56,26 @@ class LayerNorm(Norm):
 
 @register_norm("rms_norm")
 class RMSNorm(Norm):
-    """`x / sqrt(mean(x^2) + eps) * weight`, statistics in float32: the norm that only scales."""
+    """`x / sqrt(mean(x^2) + eps) * weight`, statistics in float32: the norm that only scales. With `unit_offset`
+    the checkpoint stores the weight around zero and the factor is `1 + weight` (the sum is made once, at load,
+    in float32)."""
 
     recordable = True
 
-    def __init__(self, width: int, eps: float, weight_suffix: str = ".weight"):
+    def __init__(self, width: int, eps: float, weight_suffix: str = ".weight", unit_offset: bool = False):
         self.width, self.eps, self.weight_suffix = width, float(eps), weight_suffix
+        self.unit_offset = bool(unit_offset)
         self.weight = None
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
-        return [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector", "around_one")]
+        return [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector",
+                          "normal" if self.unit_offset else "around_one")]
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
         self.weight = tensors[prefix + self.weight_suffix]
+        if self.unit_offset:
+            self.weight = (self.weight.float() + 1.0).contiguous()
 
     def forward(self, x, want_f32: bool, want_compute: bool):
         return self.ops.layernorm(x, self.weight, None, self.eps, self.dtype, want_f32, want_compute, center=False)

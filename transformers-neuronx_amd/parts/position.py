@@ -43,6 +43,30 @@ class NoPositions(PositionEncoding):
         return self.ops.to_stream(x, self.dtype, want_compute, scale=scale)
 
 
+@register_position("sinusoidal")
+class SinusoidalPositions(PositionEncoding):
+    """Fixed sines and cosines added to the embedded tokens: element 2i of the token at position p gets
+    sin(p * base^(-2i / width)), element 2i + 1 the cosine of the same angle. No table: the kernel that starts the
+    stream makes the angles, in float32, so there is no longest request."""
+
+    recordable = True
+
+    def __init__(self, width: int, base: float = 10000.0):
+        if width % 2:
+            raise ValueError(f"sines and cosines come in pairs: the width must be even, got {width}")
+        self.width, self.base = width, float(base)
+
+    def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
+        super().load(tensors, prefix, ops, dtype)
+        import torch
+        # base^(-2i / width), made in float64 and rounded once
+        i = torch.arange(self.width // 2, dtype=torch.float64)
+        self.freqs = (self.base ** (-2.0 * i / self.width)).to(torch.float32).to(getattr(ops, "device", "cpu"))
+
+    def at_input(self, x, positions, want_compute: bool, scale: float = 1.0):
+        return self.ops.add_sinusoid(x, positions, self.freqs, self.dtype, want_compute, scale=scale)
+
+
 @register_position("rotary")
 class RotaryPositions(PositionEncoding):
     """Turns pairs of query and key elements by an angle that grows with the position: of the first `dims`

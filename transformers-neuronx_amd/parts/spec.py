@@ -30,6 +30,8 @@ class ParamDecl:
     init    how the random-weights mode draws it: 'normal' (mean 0),
             'around_one' (mean 1), 'around_half' (mean 1/2), 'around_mean' (mean 1 / its size), all with the configuration's deviation
     tied_to another tensor's name that stands in when this one is absent
+    shape   a dimension may be None: the checkpoint's tensor decides it (the part reads it off the tensor it is
+            handed); random weights cannot be drawn for such a declaration
     """
     name: str
     shape: Tuple[int, ...]

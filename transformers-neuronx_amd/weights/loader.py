@@ -157,7 +157,8 @@ def check(decls: List[ParamDecl], source, base_prefix: str = "", unread: Iterabl
         src = names[d.name]
         if src is None:
             continue
-        if tuple(source.shape(src)) != tuple(d.shape):
+        have = tuple(source.shape(src))
+        if len(have) != len(d.shape) or any(w is not None and w != h for w, h in zip(d.shape, have)):
             wrong_shape.append((src, source.shape(src), d.shape))
         dt = source.dtype(src)
         is_float = isinstance(dt, torch.dtype) and dt.is_floating_point

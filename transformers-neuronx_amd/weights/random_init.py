@@ -33,6 +33,9 @@ def random_tensors(decls: List[ParamDecl], std: float, seed: int, matrix_dtype: 
             continue
         if d.role == "index":
             raise ValueError(f"no random rule for integer table {d.name}")
+        if any(n is None for n in d.shape):
+            raise ValueError(f"tensor {d.name} has a size that only a checkpoint gives ({d.shape}): the configuration "
+                             f"must name it before random weights can be drawn")
         t = torch.randn(d.shape, generator=gen, device=device, dtype=torch.float32) * std
         if d.init == "around_one":
             t += 1.0
