@@ -30,6 +30,7 @@ struct PrepareArgs {
   long long page_stride;    // elements from one page to the next
   int num_pages, page_size;
   int heads, groups, n, v, d;
+  int per_head;             // every head is normed by itself (the weights, if any, still one a projection element)
 };
 
 // Element `e` of head `head` of a normed projection, turned by the token's position. `x` points at the
@@ -92,6 +93,26 @@ __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
   const float* x = part == 0 ? row : row + nq;
   const float* w = part == 0 ? a.q_weight : a.k_weight;
   const int count = part == 0 ? nq : nk, heads = part == 0 ? a.heads : a.groups;
+  if (a.per_head) {
+    // a wave a head: the head's sum of squares over its lanes, then its elements
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    __syncthreads();       // the token's sines and cosines are there
+    T* kp = part == 1 ? (T*)a.k_pages + (size_t)page * a.page_stride : nullptr;
+    T* q_out = part == 0 ? (T*)a.q_out + (size_t)t * a.heads * a.d : nullptr;
+    for (int head = wave; head < heads; head += 4) {
+      float s = 0.f;
+      for (int e = lane; e < a.n; e += 64) s += x[head * a.n + e] * x[head * a.n + e];
+      const float r = 1.f / sqrtf(wave_sum(s) / (float)a.n + a.eps);
+      for (int e = lane; e < a.d; e += 64) {
+        const float val = e < a.n ? turned(x, w, r, head, e, a, cosines, sines) : 0.f;
+        if (part == 0)
+          q_out[head * a.d + e] = from_f32<T>(val * a.scale);
+        else
+          kp[((size_t)head * a.page_size + off) * a.d + e] = from_f32<T>(val);
+      }
+    }
+    return;
+  }
   float norm = 1.f;
   if (w != nullptr) {
     float s = 0.f;
@@ -122,7 +143,7 @@ extern "C" int tnx_qkv_prepare(const float* proj, int ld, const float* q_weight,
                                const float* mix_weight, const float* first, long long first_ld, const int* token_page,
                                const int* token_offset, void* q_out, void* k_pages, void* v_pages, long long page_stride,
                                int num_pages, int page_size, int dtype, int tokens, int heads, int groups, int n, int v,
-                               int d, hipStream_t stream) {
+                               int d, int per_head, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && heads > 0 && groups > 0 && n > 0 && v > 0, "qkv_prepare: bad sizes");
   TNX_REQUIRE(d >= n && d >= v, "qkv_prepare: cached heads of %d elements do not hold %d and %d", d, n, v);
   TNX_REQUIRE(ld >= heads * n + groups * (n + v), "qkv_prepare: rows of %d elements, %d needed", ld,
@@ -134,7 +155,8 @@ extern "C" int tnx_qkv_prepare(const float* proj, int ld, const float* q_weight,
   TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "qkv_prepare: dtype %d", dtype);
   if (tokens == 0) return 0;
   PrepareArgs a{proj, ld, q_weight, k_weight, eps, freqs, half, interleaved, positions, scale, mix_weight, first, first_ld,
-                token_page, token_offset, q_out, k_pages, v_pages, page_stride, num_pages, page_size, heads, groups, n, v, d};
+                token_page, token_offset, q_out, k_pages, v_pages, page_stride, num_pages, page_size, heads, groups, n, v, d,
+                per_head};
   if (dtype == TNX_F32)
     qkv_prepare_kernel<float><<<dim3(tokens, 3), 256, 0, stream>>>(a);
   else

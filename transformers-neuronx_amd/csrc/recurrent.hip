@@ -1,0 +1,217 @@
+// Recurrences that carry a state of fixed size from token to token, element by element.
+//   min_gru                  S <- (1 - z) S + z c, the result S silu(g)
+//   channel_conv             a causal convolution of a few taps on every channel, with a bias and per-request state
+//   gated_linear_recurrence  S <- a S + sqrt(1 - a^2) i u with a = exp(rate sigmoid(r')), the result S gelu_tanh(y)
+// Gates, decays and state are float32 with full-precision exponentials. A thread owns one channel of one run and
+// walks its tokens; what does not depend on the state (loads, gates) is made eight tokens at a time ahead of the
+// chain. State lies by position: the token at position p reads place (p - 1) & 1 of two and writes place p & 1, so
+// a step of single tokens that is recorded and run again reads what it read the first time.
+#include "common.h"
+
+TNX_DEFINE_ERROR_API
+
+namespace {
+
+__device__ __forceinline__ float sigmoid_full(float x) { return 1.f / (1.f + expf(-x)); }
+
+constexpr int AHEAD = 8;
+
+template <typename T>
+__global__ void __launch_bounds__(256)
+min_gru_kernel(const float* __restrict__ proj, int ld, int inner, const int* __restrict__ positions,
+               const int* __restrict__ run_start, const int* __restrict__ slots, float* __restrict__ carried,
+               T* __restrict__ out, long long out_ld, float out_scale) {
+  const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  const int first = run_start[r], n = run_start[r + 1] - first;
+  if (c >= inner || n <= 0) return;
+  const int p0 = positions[first];
+  float* mine = carried + (size_t)slots[r] * 2 * inner;
+  float s = p0 > 0 ? mine[(size_t)((p0 - 1) & 1) * inner + c] : 0.f;
+  for (int i0 = 0; i0 < n; i0 += AHEAD) {
+    float z[AHEAD], cand[AHEAD], g[AHEAD];
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= n) break;
+      const float* row = proj + (size_t)(first + i0 + k) * ld;
+      z[k] = row[c];
+      cand[k] = row[inner + c];
+      g[k] = row[2 * inner + c];
+    }
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= n) break;
+      z[k] = sigmoid_full(z[k]);
+      cand[k] = cand[k] >= 0.f ? cand[k] + 0.5f : sigmoid_full(cand[k]);
+      g[k] = g[k] * sigmoid_full(g[k]) * out_scale;
+    }
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= n) break;
+      s = (1.f - z[k]) * s + z[k] * cand[k];
+      out[(size_t)(first + i0 + k) * out_ld + c] = from_f32<T>(s * g[k]);
+    }
+  }
+  mine[(size_t)((p0 + n - 1) & 1) * inner + c] = s;
+}
+
+// u[t, c] = bias[c] + sum_j w[j, c] x[t - taps + 1 + j, c] over the tokens of t's own request (zeros before its
+// start); inputs from before the step's run come from the request's state `[taps, channels]`, the input at
+// position p at place p mod taps. Weights tap by tap, `[taps, channels]`.
+template <typename T>
+__global__ void __launch_bounds__(256)
+channel_conv_kernel(const float* __restrict__ x, long long ld, const float* __restrict__ w, const float* __restrict__ bias,
+                    const float* __restrict__ state, int taps, const int* __restrict__ positions,
+                    const int* __restrict__ token_request, const int* __restrict__ run_start,
+                    const int* __restrict__ slots, float* __restrict__ out, T* __restrict__ out_cd, int channels) {
+  const int t = blockIdx.x;
+  const int r = token_request[t];
+  const int i = t - run_start[r], p = positions[t];
+  const float* mine = state ? state + (size_t)slots[r] * taps * channels : nullptr;
+  for (int c = threadIdx.x; c < channels; c += 256) {
+    float acc = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+      const int back = taps - 1 - j;
+      float v = 0.f;
+      if (back <= i)
+        v = x[(size_t)(t - back) * ld + c];
+      else if (back <= p && mine)
+        v = mine[(size_t)((p - back) % taps) * channels + c];
+      acc = fmaf(w[(size_t)j * channels + c], v, acc);
+    }
+    out[(size_t)t * channels + c] = acc;
+    if (out_cd) out_cd[(size_t)t * channels + c] = from_f32<T>(acc);
+  }
+}
+
+__global__ void __launch_bounds__(256)
+channel_state_kernel(const float* __restrict__ x, long long ld, float* __restrict__ state, int taps,
+                     const int* __restrict__ positions, const int* __restrict__ run_start,
+                     const int* __restrict__ slots, int channels) {
+  const int r = blockIdx.y;
+  const int c = blockIdx.x * 256 + threadIdx.x;
+  const int first = run_start[r], n = run_start[r + 1] - first;
+  if (c >= channels || n == 0) return;
+  float* mine = state + (size_t)slots[r] * taps * channels;
+  for (int i = max(0, n - (taps - 1)); i < n; ++i)
+    mine[(size_t)(positions[first + i] % taps) * channels + c] = x[(size_t)(first + i) * ld + c];
+}
+
+struct RecurrenceArgs {
+  const float* gates;       // [T, blocks, 2 w]
+  const float* gate_bias;   // [blocks, 2 w]
+  const float* u;           // [T, channels]
+  const float* y;           // [T, y_ld]
+  long long y_ld;
+  const float* rate;        // [channels]
+  const int* positions;
+  const int* run_start;
+  const int* slots;
+  float* carried;           // [slots, 2, channels]
+  void* out;
+  long long out_ld;
+  float out_scale;
+  int channels, w;
+};
+
+template <typename T>
+__global__ void __launch_bounds__(256) gated_linear_recurrence_kernel(RecurrenceArgs a) {
+  const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  const int first = a.run_start[r], n = a.run_start[r + 1] - first;
+  if (c >= a.channels || n <= 0) return;
+  const int b = c / a.w, j = c - b * a.w;
+  const int at_r = b * 2 * a.w + j, at_i = at_r + a.w;            // within a token's gates
+  const float bias_r = a.gate_bias[at_r], bias_i = a.gate_bias[at_i], rate = a.rate[c];
+  const int p0 = a.positions[first];
+  float* mine = a.carried + (size_t)a.slots[r] * 2 * a.channels;
+  float s = p0 > 0 ? mine[(size_t)((p0 - 1) & 1) * a.channels + c] : 0.f;
+  T* out = (T*)a.out;
+  const size_t gates_ld = (size_t)2 * a.channels;
+  for (int i0 = 0; i0 < n; i0 += AHEAD) {
+    float decay[AHEAD], inp[AHEAD], y[AHEAD];
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= n) break;
+      const size_t t = (size_t)(first + i0 + k);
+      decay[k] = a.gates[t * gates_ld + at_r];
+      inp[k] = a.gates[t * gates_ld + at_i];
+      y[k] = a.y[t * a.y_ld + c];
+    }
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= n) break;
+      const float uv = a.u[(size_t)(first + i0 + k) * a.channels + c];
+      const float av = expf(rate * sigmoid_full(decay[k] + bias_r));
+      decay[k] = av;
+      inp[k] = sqrtf(1.f - av * av) * sigmoid_full(inp[k] + bias_i) * uv;
+      y[k] = apply_act(y[k], TNX_ACT_GELU_NEW) * a.out_scale;
+    }
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= n) break;
+      s = decay[k] * s + inp[k];
+      out[(size_t)(first + i0 + k) * a.out_ld + c] = from_f32<T>(s * y[k]);
+    }
+  }
+  mine[(size_t)((p0 + n - 1) & 1) * a.channels + c] = s;
+}
+
+}  // namespace
+
+extern "C" int tnx_min_gru(const float* proj, int ld, int inner, const int* positions, const int* run_start,
+                           const int* slots, float* carried, void* out, long long out_ld, int out_dtype, float out_scale,
+                           int tokens, int runs, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && runs >= 0 && inner > 0 && ld >= 3 * inner && out_ld >= inner, "min_gru: bad sizes");
+  TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "min_gru: dtype %d", out_dtype);
+  if (tokens == 0 || runs == 0) return 0;
+  const dim3 grid((inner + 255) / 256, runs);
+  if (out_dtype == TNX_F32)
+    min_gru_kernel<float><<<grid, 256, 0, stream>>>(proj, ld, inner, positions, run_start, slots, carried, (float*)out,
+                                                    out_ld, out_scale);
+  else
+    min_gru_kernel<bf16_t><<<grid, 256, 0, stream>>>(proj, ld, inner, positions, run_start, slots, carried, (bf16_t*)out,
+                                                     out_ld, out_scale);
+  TNX_CHECK_LAUNCH("min_gru");
+  return 0;
+}
+
+extern "C" int tnx_channel_conv(const float* x, long long ld, const float* w, const float* bias, float* state, int taps,
+                                const int* positions, const int* token_request, const int* run_start, const int* slots,
+                                float* out, void* out_cd, int cd_dtype, int tokens, int channels, int runs,
+                                hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && channels > 0 && taps >= 1 && runs >= 0 && ld >= channels, "channel_conv: bad sizes");
+  TNX_REQUIRE(taps == 1 || state, "channel_conv: %d taps need the requests' state", taps);
+  if (tokens == 0) return 0;
+  if (out_cd && cd_dtype == TNX_BF16)
+    channel_conv_kernel<bf16_t><<<tokens, 256, 0, stream>>>(x, ld, w, bias, taps > 1 ? state : nullptr, taps, positions,
+                                                            token_request, run_start, slots, out, (bf16_t*)out_cd, channels);
+  else
+    channel_conv_kernel<float><<<tokens, 256, 0, stream>>>(x, ld, w, bias, taps > 1 ? state : nullptr, taps, positions,
+                                                           token_request, run_start, slots, out, nullptr, channels);
+  TNX_CHECK_LAUNCH("channel_conv");
+  if (taps > 1) {
+    channel_state_kernel<<<dim3((channels + 255) / 256, runs), 256, 0, stream>>>(x, ld, state, taps, positions, run_start,
+                                                                                slots, channels);
+    TNX_CHECK_LAUNCH("channel_state");
+  }
+  return 0;
+}
+
+extern "C" int tnx_gated_linear_recurrence(const float* gates, const float* gate_bias, const float* u, const float* y,
+                                           long long y_ld, const float* rate, const int* positions, const int* run_start,
+                                           const int* slots, float* carried, void* out, long long out_ld, int out_dtype,
+                                           float out_scale, int tokens, int runs, int blocks, int w, hipStream_t stream) {
+  TNX_REQUIRE(tokens >= 0 && runs >= 0 && blocks > 0 && w > 0, "gated_linear_recurrence: bad sizes");
+  const int channels = blocks * w;
+  TNX_REQUIRE(y_ld >= channels && out_ld >= channels, "gated_linear_recurrence: rows shorter than %d", channels);
+  TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "gated_linear_recurrence: dtype %d", out_dtype);
+  if (tokens == 0 || runs == 0) return 0;
+  RecurrenceArgs a{gates, gate_bias, u, y, y_ld, rate, positions, run_start, slots, carried, out, out_ld, out_scale,
+                   channels, w};
+  const dim3 grid((channels + 255) / 256, runs);
+  if (out_dtype == TNX_F32)
+    gated_linear_recurrence_kernel<float><<<grid, 256, 0, stream>>>(a);
+  else
+    gated_linear_recurrence_kernel<bf16_t><<<grid, 256, 0, stream>>>(a);
+  TNX_CHECK_LAUNCH("gated_linear_recurrence");
+  return 0;
+}

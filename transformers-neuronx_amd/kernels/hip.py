@@ -119,7 +119,8 @@ _SIGNATURES = {
     "prepare": {
         "tnx_qkv_prepare": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_void_p,
                             _c_float, _c_void_p, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
-                            _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                            _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                            _c_void_p],
     },
     "memory": {
         "tnx_matrix_memory": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
@@ -135,6 +136,26 @@ _SIGNATURES = {
         "tnx_expert_order": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                              _c_void_p, _c_void_p],
         "tnx_expert_combine": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "hyper": {
+        "tnx_add_sinusoid": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int,
+                             _c_float, _c_void_p],
+        "tnx_hyper_step": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p,
+                           _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "recurrent": {
+        "tnx_min_gru": [_c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_ll, _c_int,
+                        _c_float, _c_int, _c_int, _c_void_p],
+        "tnx_channel_conv": [_c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                             _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_gated_linear_recurrence": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_ll, _c_void_p, _c_void_p,
+                                        _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_ll, _c_int, _c_float, _c_int,
+                                        _c_int, _c_int, _c_int, _c_void_p],
+    },
+    "scored": {
+        "tnx_attention_scored": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                 _c_int, _c_void_p, _c_ll, _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float,
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "probe": {
         "tnx_probe_stream_read": [_c_void_p, ctypes.c_size_t, _c_void_p, _c_int, _c_void_p],
@@ -1378,11 +1399,14 @@ class HipOps:
     # ---------------------------------------------------------------- normed, turned and blended projections
 
     def qkv_prepare(self, proj, num_heads, num_kv, head_size, value_size, cache_head, q_weight, k_weight, eps, freqs,
-                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages):
-        """See `ReferenceOps.qkv_prepare`."""
+                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages, per_head=False):
+        """See `ReferenceOps.qkv_prepare`. The rows of `proj` may hold more behind the values."""
         t = ctx.num_tokens
-        total = num_heads * head_size + num_kv * (head_size + value_size)
-        _want(proj, "projections", torch.float32, (t, total))
+        need = num_heads * head_size + num_kv * (head_size + value_size)
+        _want(proj, "projections", torch.float32)
+        if proj.dim() != 2 or proj.shape[0] != t or proj.shape[1] < need:
+            raise ValueError(f"projections must be [{t}, {need} or more], got {tuple(proj.shape)}")
+        total = proj.shape[1]
         if q_weight is not None:
             _want(q_weight, "query norm", torch.float32, (num_heads * head_size,))
             _want(k_weight, "key norm", torch.float32, (num_kv * head_size,))
@@ -1405,9 +1429,171 @@ class HipOps:
                    float(scale), _ptr(mix_weight) if first_values is not None else None, _ptr(first_values), first_ld,
                    _ptr(view.token_page), _ptr(view.token_offset), _ptr(q), _ptr(k_pages), _ptr(v_pages),
                    k_pages.stride(0), num_pages, view.page_size, _code(self.dtype), t, num_heads, num_kv, head_size,
-                   value_size, cache_head, _stream(),
+                   value_size, cache_head, int(bool(per_head)), _stream(),
                    work=(f"{t}x{total}", t * (total * 4 + (num_heads + 2 * num_kv) * cache_head * q.element_size()), 0.0))
         return q
+
+    # ---------------------------------------------------------------- several copies of the stream
+
+    def add_sinusoid(self, src, positions, freqs, dtype, want_compute, scale=1.0):
+        """See `ReferenceOps.add_sinusoid`."""
+        _want(src, "src")
+        t, width = src.shape
+        _want(positions, "positions", torch.int32, (t,))
+        _want(freqs, "frequencies", torch.float32, (width // 2,))
+        out = torch.empty(t, width, dtype=torch.float32, device=src.device)
+        cd = torch.empty(t, width, dtype=dtype, device=src.device) if want_compute and dtype != torch.float32 else None
+        self._call("hyper", "tnx_add_sinusoid", _ptr(src), _code(src.dtype), _ptr(positions), _ptr(freqs), _ptr(out),
+                   _ptr(cd), _code(dtype), t, width, float(scale), _stream(),
+                   work=(f"{t}x{width}", t * width * (4 + src.element_size()), 0.0))
+        return out, ((cd if cd is not None else out) if want_compute else None)
+
+    def _hyper(self, copies, pending, read, norm_weight, eps, h32, hcd, total):
+        _want(copies, "copies of the stream", torch.float32)
+        s, t, width = copies.shape
+        y = mix = out_w = None
+        if pending is not None:
+            y, mix, out_w = pending
+            _want(y, "the result to join", torch.float32, (t, width))
+            _want(mix, "mix", torch.float32, (s, s))
+            _want(out_w, "out", torch.float32, (s,))
+        if read is not None:
+            _want(read, "in", torch.float32, (s,))
+            _want(norm_weight, "norm weight", torch.float32, (width,))
+        moved = s * t * width * 4.0 * (2 if pending is not None else 1) + (t * width * 4.0 if pending is not None else 0)
+        self._call("hyper", "tnx_hyper_step", _ptr(copies), _ptr(y), _ptr(mix), _ptr(out_w), _ptr(read), _ptr(norm_weight),
+                   float(eps), _ptr(h32), _ptr(hcd), _code(hcd.dtype) if hcd is not None else 0, _ptr(total), s, t, width,
+                   _stream(), work=(f"{s}x{t}x{width}", moved + t * width * 4.0, 0.0))
+
+    def hyper_step(self, copies, pending, read, norm_weight, eps, dtype, want_f32, want_compute):
+        """See `ReferenceOps.hyper_step`."""
+        _, t, width = copies.shape
+        same = dtype == torch.float32
+        h32 = torch.empty(t, width, dtype=torch.float32, device=copies.device) if (want_f32 or (want_compute and same)) else None
+        hcd = torch.empty(t, width, dtype=dtype, device=copies.device) if (want_compute and not same) else None
+        self._hyper(copies, pending, read, norm_weight, eps, h32, hcd, None)
+        return (h32 if want_f32 else None), ((h32 if same else hcd) if want_compute else None)
+
+    def hyper_sum(self, copies, pending):
+        """See `ReferenceOps.hyper_sum`."""
+        _, t, width = copies.shape
+        total = torch.empty(t, width, dtype=torch.float32, device=copies.device)
+        self._hyper(copies, pending, None, None, 0.0, None, None, total)
+        return total
+
+    # ---------------------------------------------------------------- scores that are not the plain ones
+
+    @staticmethod
+    def _rows_apart(x, name, dtype, t, width):
+        """A `[t, width]` tensor whose rows may lie apart (a slice of columns): its row distance in elements."""
+        if (not x.is_cuda or x.dtype != dtype or x.dim() != 2 or tuple(x.shape) != (t, width)
+                or (width > 1 and x.stride(1) != 1)):
+            raise ValueError(f"{name} must be {dtype} [{t}, {width}] with dense rows on the GPU, got {tuple(x.shape)} {x.dtype}")
+        return x.stride(0) if t > 1 else max(x.stride(0), width)
+
+    def attention_scored(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None,
+                         chunk=None, softcap=None, distance_bias=None, gate=None, value_size=None, out=None,
+                         out_scale=1.0):
+        """See `ReferenceOps.attention_scored`."""
+        t = ctx.num_tokens
+        value_size = head_size if value_size is None else value_size
+        _want(q, "q", self.dtype, (t, num_heads * head_size))
+        num_pages = self._check_pages(k_pages, v_pages, num_kv_heads, head_size, view.page_size)
+        _want(view.block_table, "block table", torch.int32, (ctx.num_requests, view.width))
+        if ctx.max_total > view.width * view.page_size:
+            raise ValueError("a request is longer than its block table")
+        if out is None:
+            out = torch.empty_like(q)
+        out_ld = self._rows_apart(out, "the result", self.dtype, t, num_heads * head_size)
+        gate_ld = self._rows_apart(gate, "the gate", torch.float32, t, num_heads * value_size) if gate is not None else 0
+        far = 0
+        if distance_bias is not None:
+            _want(distance_bias, "bias by distance", torch.float32)
+            if distance_bias.dim() != 2 or distance_bias.shape[0] != num_heads:
+                raise ValueError(f"the bias by distance is [heads, distances], got {tuple(distance_bias.shape)}")
+            far = distance_bias.shape[1] - 1
+        pad = self._page_pad(k_pages, num_kv_heads, head_size, view.page_size)
+        self._call("scored", "tnx_attention_scored", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
+                   _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
+                   num_pages, _ptr(out), out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far,
+                   float(softcap or 0.0), int(window or 0), int(chunk or 0), t, num_heads, num_kv_heads, head_size,
+                   value_size, pad, _stream(),
+                   work=self._scored_work(ctx, num_heads, num_kv_heads, head_size, window, chunk, q.element_size())
+                   if debug.timer() is not None else None)
+        return out
+
+    @staticmethod
+    def _scored_work(ctx, num_heads, num_kv_heads, head_size, window, chunk, item):
+        """For a kernel timer: the keys the step's queries see (a query at position p sees p + 1, cut by the window
+        and by the chunk it lies in), the bytes of keys and values its runs must read once, the flops."""
+        lens, cached = ctx.run_lens_host.astype(np.int64), ctx.cached_lens_host.astype(np.int64)
+        pairs, span = 0.0, 0.0
+        for n, have in zip(lens, cached):
+            p = np.arange(have, have + n, dtype=np.int64)
+            seen = p + 1
+            if window:
+                seen = np.minimum(seen, window)
+            if chunk:
+                seen = np.minimum(seen, p % chunk + 1)
+            pairs += float(seen.sum())
+            first = int((p - seen + 1).min()) if n else 0
+            span += float(have + n - first)
+        return (f"{len(lens)} runs {int(lens.sum())} tokens", span * 2 * num_kv_heads * head_size * item,
+                4.0 * num_heads * head_size * pairs)
+
+    # ---------------------------------------------------------------- recurrences
+
+    def min_gru(self, proj, inner, ctx, carried, out=None, out_scale=1.0):
+        """See `ReferenceOps.min_gru`."""
+        t = ctx.num_tokens
+        _want(proj, "projections", torch.float32, (t, 3 * inner))
+        _want(carried, "carried state", torch.float32, (carried.shape[0], 2, inner))
+        if out is None:
+            out = torch.empty(t, inner, dtype=self.dtype, device=proj.device)
+        out_ld = self._rows_apart(out, "the result", self.dtype, t, inner)
+        self._call("recurrent", "tnx_min_gru", _ptr(proj), 3 * inner, inner, _ptr(ctx.positions), _ptr(ctx.run_start),
+                   _ptr(ctx.slots), _ptr(carried), _ptr(out), out_ld, _code(self.dtype), float(out_scale), t,
+                   ctx.num_requests, _stream(), work=(f"{t}x{inner}", t * inner * (12.0 + out.element_size()), 0.0))
+        return out
+
+    def channel_conv(self, x, weight, bias, ctx, state):
+        """See `ReferenceOps.channel_conv`."""
+        t = ctx.num_tokens
+        channels, taps = weight.shape
+        ld = self._rows_apart(x, "the convolution's input", torch.float32, t, channels)
+        _want(weight, "convolution weights", torch.float32, (channels, taps))
+        _want(bias, "convolution bias", torch.float32, (channels,))
+        if taps > 1:
+            _want(state, "convolution state", torch.float32, (state.shape[0], taps, channels))
+        out = torch.empty(t, channels, dtype=torch.float32, device=x.device)
+        cd = torch.empty(t, channels, dtype=self.dtype, device=x.device) if self.dtype != torch.float32 else None
+        self._call("recurrent", "tnx_channel_conv", _ptr(x), ld, _ptr(self._taps_first(weight)), _ptr(bias),
+                   _ptr(state) if taps > 1 else None, taps, _ptr(ctx.positions), _ptr(ctx.token_request),
+                   _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(out), _ptr(cd), _code(self.dtype), t, channels,
+                   ctx.num_requests, _stream(), work=(f"{t}x{channels}", t * channels * 10.0, 0.0))
+        return out, (cd if cd is not None else out)
+
+    def gated_linear_recurrence(self, gates, gate_bias, u, y, rate, ctx, carried, out=None, out_scale=1.0):
+        """See `ReferenceOps.gated_linear_recurrence`."""
+        t = ctx.num_tokens
+        _want(gates, "gates", torch.float32)
+        if gates.dim() != 3 or gates.shape[0] != t or gates.shape[2] % 2:
+            raise ValueError(f"gates must be [{t}, blocks, 2 w], got {tuple(gates.shape)}")
+        blocks, w = gates.shape[1], gates.shape[2] // 2
+        channels = blocks * w
+        _want(gate_bias, "gate biases", torch.float32, (blocks, 2 * w))
+        _want(u, "u", torch.float32, (t, channels))
+        _want(rate, "rate", torch.float32, (channels,))
+        _want(carried, "carried state", torch.float32, (carried.shape[0], 2, channels))
+        y_ld = self._rows_apart(y, "y", torch.float32, t, channels)
+        if out is None:
+            out = torch.empty(t, channels, dtype=self.dtype, device=u.device)
+        out_ld = self._rows_apart(out, "the result", self.dtype, t, channels)
+        self._call("recurrent", "tnx_gated_linear_recurrence", _ptr(gates), _ptr(gate_bias), _ptr(u), _ptr(y), y_ld,
+                   _ptr(rate), _ptr(ctx.positions), _ptr(ctx.run_start), _ptr(ctx.slots), _ptr(carried), _ptr(out), out_ld,
+                   _code(self.dtype), float(out_scale), t, ctx.num_requests, blocks, w, _stream(),
+                   work=(f"{t}x{channels}", t * channels * (16.0 + out.element_size()), 0.0))
+        return out
 
     # ---------------------------------------------------------------- the matrix memory
 
