@@ -140,9 +140,10 @@ __global__ void __launch_bounds__(256) gated_linear_recurrence_kernel(Recurrence
     for (int k = 0; k < AHEAD; ++k) {
       if (i0 + k >= n) break;
       const float uv = a.u[(size_t)(first + i0 + k) * a.channels + c];
-      const float av = expf(rate * sigmoid_full(decay[k] + bias_r));
-      decay[k] = av;
-      inp[k] = sqrtf(1.f - av * av) * sigmoid_full(inp[k] + bias_i) * uv;
+      const float log_a = rate * sigmoid_full(decay[k] + bias_r);
+      decay[k] = expf(log_a);
+      // sqrt(1 - a^2) as sqrt(-expm1(2 log a)): no cancellation where a is close to 1
+      inp[k] = sqrtf(-expm1f(2.f * log_a)) * sigmoid_full(inp[k] + bias_i) * uv;
       y[k] = apply_act(y[k], TNX_ACT_GELU_NEW) * a.out_scale;
     }
 #pragma unroll

@@ -601,8 +601,9 @@ class ReferenceOps:
         pre = gates.float() + gate_bias.float()[None]
         r = torch.sigmoid(pre[:, :, :w]).reshape(t, blocks * w)
         i = torch.sigmoid(pre[:, :, w:]).reshape(t, blocks * w)
-        a = torch.exp(rate.float()[None, :] * r)
-        inp = torch.sqrt(1.0 - a * a) * i * u.float()
+        log_a = rate.float()[None, :] * r
+        a = torch.exp(log_a)
+        inp = torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u.float()      # sqrt(1 - a^2) without the cancellation near a = 1
         res = torch.empty(t, blocks * w, dtype=torch.float32, device=u.device)
         start = 0
         for q in range(ctx.num_requests):
