@@ -77,13 +77,35 @@ def sunatar_config(width, heads, head, ff, vocab, layers, window=1024):
                         dict(type="attention", mixer=attention, mlp=mlp) for i in range(layers)])
 
 
-# a new design beside the closest one the engine had, at equal sizes: {design: {size: (its config, the other's)}}
+def tadolix_config(width, heads, head, ff, vocab, layers, chunk=1024):
+    """config.json contents of a Tadolix model at the sizes of a published layer: four copies of the stream, a
+    convolution of four taps before every mixer; every third layer (the second first) Griffin's recurrent block of
+    the model's width in sixteen parts, the others attention in chunks (a quarter as many key/value heads as query
+    heads, capped scores, a bias by distance of 32 rows) beside a minimal gated recurrence of the model's width;
+    every layer a gated feed-forward of `ff`."""
+    pair = dict(left=dict(heads=heads, kv_heads=max(1, heads // 4), dim=head, vdim=head, scale=head ** -0.5, softcap=30.0,
+                          bias_max=chunk, bias_rows=32, mask=dict(size=chunk)), right=dict(width=width), left_scale=1.0, right_scale=1.0)
+    recurrent = dict(width=width, blocks=16, conv=4)
+    mlp = dict(kind="dense", ff=ff)
+    return dict(architecture="Tadolix", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=width ** 0.5),
+                canon=dict(taps=4), streams=4, init_std=0.02, max_positions=4096,
+                layers=[dict(type="rglru", mixer=recurrent, mlp=mlp) if i % 3 == 1 else
+                        dict(type="parallel", mixer=pair, mlp=mlp) for i in range(layers)])
+
+
+# a new design beside the closest one the engine had, at equal sizes: {design: {size: (its config, the other's)}};
+# the other's is the name of an OPT preset, or (design, its config)
 BESIDE = {"ratesun": {
     "2048 wide": (lambda n: ratesun_config(2048, 16, 8192, 50272, n, 768), "1.3b"),
     "4096 wide": (lambda n: ratesun_config(4096, 32, 16384, 50272, n, 1536), "6.7b"),
 }, "sunatar": {
     "2048 wide": (lambda n: sunatar_config(2048, 32, 64, 8192, 50272, n), "1.3b"),
     "4096 wide": (lambda n: sunatar_config(4096, 32, 128, 16384, 50272, n), "6.7b"),
+}, "tadolix": {
+    "2048 wide": (lambda n: tadolix_config(2048, 32, 64, 8192, 50272, n),
+                  ("sunatar", lambda n: sunatar_config(2048, 32, 64, 8192, 50272, n))),
+    "4096 wide": (lambda n: tadolix_config(4096, 32, 128, 16384, 50272, n),
+                  ("sunatar", lambda n: sunatar_config(4096, 32, 128, 16384, 50272, n))),
 }}
 PREFILL_TOKENS = 2048
 PEAK_HBM_GBS = 8000.0                      # MI355X, published
@@ -548,13 +570,15 @@ def beside(args):
     import torch
     layers = args.layers or 4
     context, tokens = args.context or 2048, min(args.prefill_tokens, args.context or 2048)
-    out = {"metric": f"{args.beside} beside OPT at equal sizes: decode tok/s @ batch {args.batch}, prefill tok/s @ {tokens:,} tokens",
+    others = {o[0] if isinstance(o, tuple) else "opt" for _, o in BESIDE[args.beside].values()}
+    out = {"metric": f"{args.beside} beside {' and '.join(sorted(others))} at equal sizes: decode tok/s @ batch {args.batch}, prefill tok/s @ {tokens:,} tokens",
            "unit": "tokens/s", "dtype": args.dtype, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "data": "synthetic (seeded random weights and token ids)", "layers": layers, "context": context, "sizes": {}}
     for size, (make, preset) in BESIDE[args.beside].items():
         row = {}
-        for design, raw in ((args.beside, make(layers)), ("opt", dict(PRESETS[preset], num_hidden_layers=layers,
-                                                                        max_position_embeddings=max(2048, context)))):
+        other = (preset[0], preset[1](layers)) if isinstance(preset, tuple) else (
+            "opt", dict(PRESETS[preset], num_hidden_layers=layers, max_position_embeddings=max(2048, context)))
+        for design, raw in ((args.beside, make(layers)), other):
             bench = Bench(raw, args.dtype, args.batch, context, step_tokens=tokens)
             keep_busy(bench.runner.ops, torch, 1.0)
             value, sec, read = bench.decode(args.batch, args.steps, args.warmup)

@@ -67,9 +67,10 @@ def bucket(n, rows, far):
     return min(rows - 1, half + math.floor(math.log(n / half) / math.log(far / half) * (rows - half)))
 
 
-def chunk_attention(m, w, p, h, eps):
+def chunk_attention(m, w, p, h, eps, only=None, weights=None):
     """The left half of a pair: softmax attention inside chunks, unit-norm queries and keys, capped scores, a bias
-    by distance, an output gate. Returns what the output matrix gives, `[T, D]`."""
+    by distance, an output gate. Returns what the output matrix gives, `[T, D]`. `only`: the queries to work out
+    (the other rows stay zero before the gate); `weights`: a dict that gets the softmax weights by (head, query)."""
     T = h.shape[0]
     H, G, n, v = m["heads"], m.get("kv_heads", m["heads"]), m["dim"], m["vdim"]
     q = unit_rms((h @ w[p + "q"].T).view(T, H, n), eps)
@@ -81,13 +82,15 @@ def chunk_attention(m, w, p, h, eps):
     out = torch.zeros(T, H, v, dtype=F64)
     for head in range(H):
         g = head // (H // G)
-        for i in range(T):
+        for i in (range(T) if only is None else only):
             first = (i // size) * size if size else 0
             s = torch.stack([q[i, head] @ k[j, g] for j in range(first, i + 1)]) * m.get("scale", n ** -0.5)
             if cap:
                 s = cap * torch.tanh(s / cap)
             s = s + torch.stack([rel[bucket(i - j, rel.shape[0], m["bias_max"]), head] for j in range(first, i + 1)])
             a = torch.softmax(s, 0)
+            if weights is not None:
+                weights[(head, i)] = (first, a)
             out[i, head] = (a[:, None] * val[first:i + 1, g]).sum(0)
     gate = torch.sigmoid(h @ w[p + "g"].T)
     return (out.reshape(T, H * v) * gate) @ w[p + "o"].T
