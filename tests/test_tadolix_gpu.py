@@ -227,12 +227,17 @@ def _standout(dtype, case, seed):
     dict(h=8, g=2, n=96, v=64, chunk=256, length=1000, run=300, ps=64, back=231, rows=16, far=256, scale=0.3, cap=30.0),  # a long portion over a chunk's edge
     dict(h=8, g=2, n=96, v=64, chunk=256, length=1000, run=300, ps=64, back=232, rows=16, far=256, scale=0.3, cap=30.0),
 ])
-def test_scored_attention_finds_the_key_that_stands_out(name, dtype, tol, case):
-    """Through the kernel that norms and stores and the attention kernel: queries and keys scaled to unit root
-    mean square a head, capped scores, the bias by distance, chunks, the gate."""
+@pytest.mark.parametrize("one_wave_a_query", [False, True])
+def test_scored_attention_finds_the_key_that_stands_out(name, dtype, tol, case, one_wave_a_query):
+    """Through the kernel that norms and stores and the attention kernels (in bfloat16 those on the matrix unit,
+    and the general one when told to): queries and keys scaled to unit root mean square a head, capped scores,
+    the bias by distance, chunks, the gate."""
+    if one_wave_a_query and dtype == torch.float32:
+        pytest.skip("float32 runs on the general kernel anyway")
     from transformers_neuronx_amd.kernels.attention_plan import attention_plan
     from transformers_neuronx_amd.parts.mixer import bias_by_distance
     ops = _ops(dtype)
+    ops.force_plain_attention = one_wave_a_query
     case = dict(case, eps=1e-4)
     h, g, n, v, length, run, ps = (case[k] for k in ("h", "g", "n", "v", "length", "run", "ps"))
     d = -(-max(n, v) // 16) * 16
@@ -260,6 +265,52 @@ def test_scored_attention_finds_the_key_that_stands_out(name, dtype, tol, case):
                                    distance_bias=bias, gate=rows[:, nq:], value_size=v, out_scale=1.0)
     # in bfloat16 the unit-norm queries and keys are rounded: scores of a few units move by hundredths
     _close(got.view(run, h, d)[:, :, :v].reshape(run, h * v), want, tol if dtype == torch.float32 else 4e-2)
+
+
+@pytest.mark.parametrize("pad", [0, 2, 3])
+def test_scored_attention_of_a_mixed_step_into_columns_of_a_wider_buffer(pad):
+    """Runs of one token (each key/value head's query heads side by side, 20 of them: two blocks of columns)
+    beside a portion and a whole prompt in one step, written times a factor into a slice of a buffer whose rows
+    are not multiples of 8 bytes apart; against the general kernel, and the columns beside the slice untouched."""
+    from transformers_neuronx_amd.kernels.attention_plan import attention_plan
+    from transformers_neuronx_amd.parts.mixer import bias_by_distance
+    h, g, n, v, d, ps = 40, 2, 32, 24, 32, 16
+    gen = torch.Generator().manual_seed(3)
+    rel = torch.randn(10, h, generator=gen)
+    bias = bias_by_distance(rel, 50).to(DEV)
+    lens, runs = [150, 97, 200, 31], [1, 1, 40, 31]
+    pages = sum(-(-n_ // ps) for n_ in lens)
+    order = torch.randperm(pages + 2, generator=gen).tolist()
+    tables, at = [], 0
+    for n_ in lens:
+        k = -(-n_ // ps)
+        tables.append(order[at:at + k] + [-1] * (13 - k))
+        at += k
+    results = {}
+    for plain in (False, True):
+        ops = _ops(torch.bfloat16)
+        ops.force_plain_attention = plain
+        k_pages = torch.zeros(pages + 2, g, ps, d, dtype=torch.bfloat16, device=DEV)
+        v_pages = torch.zeros(pages + 2, g, d, ps, dtype=torch.bfloat16, device=DEV)
+        gen2 = torch.Generator().manual_seed(4)
+        width = h * n + g * (n + v) + h * v
+        for heads, cached in (([n_ - r for n_, r in zip(lens, runs)], [0] * 4), (runs, [n_ - r for n_, r in zip(lens, runs)])):
+            if not any(heads):
+                continue
+            live = [i for i, t in enumerate(heads) if t]
+            ctx = _ctx([heads[i] for i in live], [cached[i] for i in live], live, {"g": [tables[i] for i in live]}, ps,
+                       {"attention": attention_plan})
+            rows = (torch.randn(sum(heads), width, generator=gen2) * 1.5).to(DEV)
+            q = ops.qkv_prepare(rows, h, g, n, v, d, None, None, 1e-5, None, False, 0.4, None, None, ctx, ctx.groups["g"],
+                                k_pages, v_pages, per_head=True)
+            both = torch.full((sum(heads), pad + h * d + 5), 7.0, dtype=torch.bfloat16, device=DEV)
+            ops.attention_scored(q, h, g, d, ctx, ctx.groups["g"], k_pages, v_pages, chunk=64, softcap=15.0,
+                                 distance_bias=bias, gate=rows[:, h * n + g * (n + v):], value_size=v,
+                                 out=both[:, pad:pad + h * d], out_scale=0.6)
+        results[plain] = both.float().cpu()
+    assert float(results[False][:, :pad].min() if pad else 7.0) == 7.0 and float(results[False][:, pad + h * d:].min()) == 7.0
+    err = float((results[False] - results[True]).abs().max() / results[True][:, pad:pad + h * d].abs().max())
+    assert err < 2e-2, err
 
 
 # ---------------------------------------------------------------- the engine

@@ -153,6 +153,10 @@ _SIGNATURES = {
                                         _c_int, _c_int, _c_int, _c_void_p],
     },
     "scored": {
+        "tnx_attention_scored_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                      _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_ll,
+                                      _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_int,
+                                      _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_scored": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_ll, _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -1513,13 +1517,23 @@ class HipOps:
                 raise ValueError(f"the bias by distance is [heads, distances], got {tuple(distance_bias.shape)}")
             far = distance_bias.shape[1] - 1
         pad = self._page_pad(k_pages, num_kv_heads, head_size, view.page_size)
+        work = (self._scored_work(ctx, num_heads, num_kv_heads, head_size, window, chunk, q.element_size())
+                if debug.timer() is not None else None)
+        if self.dtype == torch.bfloat16 and not self.force_plain_attention and "tile_run" in ctx.plan:
+            # on the matrix unit: the runs of several tokens by tiles of queries, the runs of one token by key/value head
+            tiles, single = ctx.plan["tile_run"], ctx.plan["decode_runs"]
+            self._call("scored", "tnx_attention_scored_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.run_start),
+                       _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size, num_pages, _ptr(tiles),
+                       _ptr(ctx.plan["tile_start"]), tiles.numel(), QUERY_TILE, _ptr(single), single.numel(), _ptr(out),
+                       out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far, float(softcap or 0.0),
+                       int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size, value_size, pad, _stream(),
+                       work=work)
+            return out
         self._call("scored", "tnx_attention_scored", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
                    num_pages, _ptr(out), out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far,
                    float(softcap or 0.0), int(window or 0), int(chunk or 0), t, num_heads, num_kv_heads, head_size,
-                   value_size, pad, _stream(),
-                   work=self._scored_work(ctx, num_heads, num_kv_heads, head_size, window, chunk, q.element_size())
-                   if debug.timer() is not None else None)
+                   value_size, pad, _stream(), work=work)
         return out
 
     @staticmethod
