@@ -3,7 +3,7 @@
 //   hyper_step     joins a sublayer's result to the copies, x_b <- sum_a mix[a, b] x_a + out[b] y, then makes the
 //                  next sublayer's input, norm(sum_a in[a] x_a), and / or the sum of the copies: one launch
 // Copies, sums and norms are float32. One block a token; a token's elements of all copies pass through the
-// block's registers once.
+// block's registers once. The number of copies is a template parameter (1 to 8).
 #include "common.h"
 
 TNX_DEFINE_ERROR_API
@@ -48,63 +48,126 @@ struct HyperArgs {
   int s, tokens, width;
 };
 
-// PER elements a thread (width <= 256 * PER): the weighted sum u stays in registers between the pass that makes
-// it and the pass that scales it.
-template <int PER>
+// S copies, PER groups of VEC consecutive elements a thread (width <= 256 * PER * VEC): every loop over the copies
+// is unrolled, so that a token's elements and the weighted sum u stay in registers between the pass that makes
+// them and the pass that scales them. VEC = 4 reads and writes 16 bytes at a time (widths that are multiples of 4).
+template <int S, int PER, int VEC>
 __global__ void __launch_bounds__(256) hyper_step_kernel(HyperArgs a) {
   __shared__ float scratch[4];
-  __shared__ float w_mix[MAX_COPIES * MAX_COPIES], w_out[MAX_COPIES], w_read[MAX_COPIES];
-  const int t = blockIdx.x, s = a.s;
-  if (threadIdx.x < s * s && a.y) w_mix[threadIdx.x] = a.mix[threadIdx.x];
-  if (threadIdx.x < s) {
-    if (a.y) w_out[threadIdx.x] = a.out_w[threadIdx.x];
-    if (a.read) w_read[threadIdx.x] = a.read[threadIdx.x];
+  const int t = blockIdx.x;
+  float w_mix[S][S], w_out[S], w_read[S];
+#pragma unroll
+  for (int c = 0; c < S; ++c) {
+    w_out[c] = a.y ? a.out_w[c] : 0.f;
+    w_read[c] = a.read ? a.read[c] : 0.f;
+#pragma unroll
+    for (int b = 0; b < S; ++b) w_mix[c][b] = a.y ? a.mix[c * S + b] : 0.f;
   }
-  __syncthreads();
   const size_t row = (size_t)t * a.width, plane = (size_t)a.tokens * a.width;
-  float u[PER];
+  float u[PER][VEC];
   float sq = 0.f;
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const int d = threadIdx.x + 256 * k;
-    u[k] = 0.f;
+    const int d = (threadIdx.x + 256 * k) * VEC;
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) u[k][e] = 0.f;
     if (d >= a.width) continue;
-    float x[MAX_COPIES];
-    for (int c = 0; c < s; ++c) x[c] = a.copies[c * plane + row + d];
-    if (a.y) {
-      const float yv = a.y[row + d];
-      float nx[MAX_COPIES];
-      for (int b = 0; b < s; ++b) {
-        float v = 0.f;
-        for (int c = 0; c < s; ++c) v = fmaf(w_mix[c * s + b], x[c], v);
-        nx[b] = fmaf(w_out[b], yv, v);
+    float x[S][VEC], yv[VEC];
+#pragma unroll
+    for (int c = 0; c < S; ++c) {
+      if (VEC == 4) {
+        const f32x4 v = *(const f32x4*)(a.copies + c * plane + row + d);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[c][e] = v[e];
+      } else {
+        x[c][0] = a.copies[c * plane + row + d];
       }
-      for (int b = 0; b < s; ++b) {
-        x[b] = nx[b];
-        a.copies[b * plane + row + d] = nx[b];
+    }
+    if (a.y) {
+      if (VEC == 4) {
+        const f32x4 v = *(const f32x4*)(a.y + row + d);
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) yv[e] = v[e];
+      } else {
+        yv[0] = a.y[row + d];
+      }
+      float nx[S][VEC];
+#pragma unroll
+      for (int b = 0; b < S; ++b)
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float v = 0.f;
+#pragma unroll
+          for (int c = 0; c < S; ++c) v = fmaf(w_mix[c][b], x[c][e], v);
+          nx[b][e] = fmaf(w_out[b], yv[e], v);
+        }
+#pragma unroll
+      for (int b = 0; b < S; ++b) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[b][e] = nx[b][e];
+        if (VEC == 4)
+          *(f32x4*)(a.copies + b * plane + row + d) = (f32x4){nx[b][0], nx[b][VEC > 1 ? 1 : 0], nx[b][VEC > 2 ? 2 : 0], nx[b][VEC > 3 ? 3 : 0]};
+        else
+          a.copies[b * plane + row + d] = nx[b][0];
       }
     }
     if (a.sum) {
-      float v = 0.f;
-      for (int c = 0; c < s; ++c) v += x[c];
-      a.sum[row + d] = v;
+      float v[VEC];
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        v[e] = 0.f;
+#pragma unroll
+        for (int c = 0; c < S; ++c) v[e] += x[c][e];
+      }
+      if (VEC == 4)
+        *(f32x4*)(a.sum + row + d) = (f32x4){v[0], v[VEC > 1 ? 1 : 0], v[VEC > 2 ? 2 : 0], v[VEC > 3 ? 3 : 0]};
+      else
+        a.sum[row + d] = v[0];
     }
     if (a.read) {
-      float v = 0.f;
-      for (int c = 0; c < s; ++c) v = fmaf(w_read[c], x[c], v);
-      u[k] = v;
-      sq = fmaf(v, v, sq);
+#pragma unroll
+      for (int e = 0; e < VEC; ++e) {
+        float v = 0.f;
+#pragma unroll
+        for (int c = 0; c < S; ++c) v = fmaf(w_read[c], x[c][e], v);
+        u[k][e] = v;
+        sq = fmaf(v, v, sq);
+      }
     }
   }
   if (!a.read) return;
   const float r = 1.f / sqrtf(block_sum<4>(sq, scratch) / (float)a.width + a.eps);
 #pragma unroll
   for (int k = 0; k < PER; ++k) {
-    const int d = threadIdx.x + 256 * k;
+    const int d = (threadIdx.x + 256 * k) * VEC;
     if (d >= a.width) continue;
-    const float h = u[k] * r * a.norm_w[d];
-    if (a.h32) a.h32[row + d] = h;
-    if (a.hcd) store_any(a.hcd, a.cd_dtype, row + d, h);
+#pragma unroll
+    for (int e = 0; e < VEC; ++e) {
+      const float h = u[k][e] * r * a.norm_w[d + e];
+      if (a.h32) a.h32[row + d + e] = h;
+      if (a.hcd) store_any(a.hcd, a.cd_dtype, row + d + e, h);
+    }
+  }
+}
+
+template <int S>
+void launch_hyper_step(const HyperArgs& a, hipStream_t stream) {
+  const bool aligned = (((uintptr_t)a.copies | (uintptr_t)a.y | (uintptr_t)a.sum) & 15) == 0;
+  const bool by_four = aligned && a.width % 4 == 0 && a.width <= 256 * 16 * 4;
+  const int per = by_four ? (a.width / 4 + 255) / 256 : (a.width + 255) / 256;
+  if (by_four) {
+    if (per <= 1)
+      hyper_step_kernel<S, 1, 4><<<a.tokens, 256, 0, stream>>>(a);
+    else if (per <= 4)
+      hyper_step_kernel<S, 4, 4><<<a.tokens, 256, 0, stream>>>(a);
+    else
+      hyper_step_kernel<S, 16, 4><<<a.tokens, 256, 0, stream>>>(a);
+  } else if (per <= 4) {
+    hyper_step_kernel<S, 4, 1><<<a.tokens, 256, 0, stream>>>(a);
+  } else if (per <= 16) {
+    hyper_step_kernel<S, 16, 1><<<a.tokens, 256, 0, stream>>>(a);
+  } else {
+    hyper_step_kernel<S, 64, 1><<<a.tokens, 256, 0, stream>>>(a);
   }
 }
 
@@ -128,15 +191,16 @@ extern "C" int tnx_hyper_step(float* copies, const float* y, const float* mix, c
   TNX_REQUIRE(!read || (norm_w && (h32 || hcd)), "hyper_step: an input needs its norm and a place");
   if (tokens == 0) return 0;
   HyperArgs a{copies, y, mix, out_w, read, norm_w, eps, h32, hcd, cd_dtype, sum, s, tokens, width};
-  const int per = (width + 255) / 256;
-  if (per <= 2)
-    hyper_step_kernel<2><<<tokens, 256, 0, stream>>>(a);
-  else if (per <= 8)
-    hyper_step_kernel<8><<<tokens, 256, 0, stream>>>(a);
-  else if (per <= 32)
-    hyper_step_kernel<32><<<tokens, 256, 0, stream>>>(a);
-  else
-    hyper_step_kernel<64><<<tokens, 256, 0, stream>>>(a);
+  switch (s) {
+    case 1: launch_hyper_step<1>(a, stream); break;
+    case 2: launch_hyper_step<2>(a, stream); break;
+    case 3: launch_hyper_step<3>(a, stream); break;
+    case 4: launch_hyper_step<4>(a, stream); break;
+    case 5: launch_hyper_step<5>(a, stream); break;
+    case 6: launch_hyper_step<6>(a, stream); break;
+    case 7: launch_hyper_step<7>(a, stream); break;
+    default: launch_hyper_step<8>(a, stream); break;
+  }
   TNX_CHECK_LAUNCH("hyper_step");
   return 0;
 }

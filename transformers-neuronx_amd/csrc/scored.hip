@@ -167,30 +167,71 @@ __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __re
   const float cap = a.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
   const bool biased = a.bias != nullptr;
 
-  for (int tile0 = tile_begin; tile0 <= last_q; tile0 += tile_step) {
-    f32x4 s[4][NQB];
+  // A tile's keys as the A operand of the scores (row r of block kb is key 16 kb + r) and its values as that
+  // of the result (row r of block db is element 16 db + r; keys 16 tb + 4 g .. + 3), zeros for what has no page,
+  // lies beyond the head's size or beyond the request.
+  bf16x8 kf[4][NKS];
+  bf16x4 vf[NDB][4];
+  auto load_keys = [&](int tile0) {
 #pragma unroll
     for (int kb = 0; kb < 4; ++kb) {
       const int key0 = tile0 + 16 * kb;
-      f32x4 acc[NQB];
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb) acc[qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
       int page = -1;
       if (key0 <= last_q) page = tab[key0 / page_size];
-      if (page >= 0 && page < num_pages) {
-        const bf16_t* kbase =
-            k_pages + (size_t)page * page_stride + ((size_t)kvh * page_size + key0 % page_size + r) * head_size;
+      const bool ok = page >= 0 && page < num_pages;
+      const bf16_t* kbase = k_pages + (size_t)(ok ? page : 0) * page_stride +
+                            ((size_t)kvh * page_size + key0 % page_size + r) * head_size;
 #pragma unroll
-        for (int ks = 0; ks < NKS; ++ks) {
-          const int d0 = 32 * ks + 8 * g;
-          const bf16x8 kf = d0 < head_size ? *(const bf16x8*)(kbase + d0) : zero8;
-#pragma unroll
-          for (int qb = 0; qb < NQB; ++qb) acc[qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qb][ks], acc[qb], 0, 0, 0);
-        }
+      for (int ks = 0; ks < NKS; ++ks) {
+        const int d0 = 32 * ks + 8 * g;
+        kf[kb][ks] = (ok && d0 < head_size) ? *(const bf16x8*)(kbase + d0) : zero8;
       }
-#pragma unroll
-      for (int qb = 0; qb < NQB; ++qb) s[kb][qb] = acc[qb];
     }
+  };
+  auto load_values = [&](int tile0) {
+#pragma unroll
+    for (int tb = 0; tb < 4; ++tb) {
+      const int key0 = tile0 + 16 * tb;
+      int page = -1;
+      if (key0 <= last_q) page = tab[key0 / page_size];
+      const bool ok = page >= 0 && page < num_pages;
+      const bf16_t* vbase = v_pages + (size_t)(ok ? page : 0) * page_stride + (size_t)kvh * head_size * page_size +
+                            key0 % page_size + 4 * g;
+      const bool tail = key0 + 16 > total;      // some keys of this block lie beyond the request
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        bf16x4 v4 = {0, 0, 0, 0};
+        if (ok && db < ndb) v4 = *(const bf16x4*)(vbase + (size_t)(16 * db + r) * page_size);
+        if (tail) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (key0 + 4 * g + i >= total) v4[i] = 0;
+        }
+        vf[db][tb] = v4;
+      }
+    }
+  };
+  // Where the registers hold both (heads of up to 128 elements), a tile's values are asked for before its
+  // scores are made and the next tile's keys as soon as they are: both arrive while the scores are capped,
+  // biased and turned into weights.
+  constexpr bool AHEAD = NDB <= 8;
+  if (AHEAD && tile_begin <= last_q) load_keys(tile_begin);
+
+  for (int tile0 = tile_begin; tile0 <= last_q; tile0 += tile_step) {
+    f32x4 s[4][NQB];
+    if (!AHEAD) load_keys(tile0);
+    if (AHEAD) load_values(tile0);
+#pragma unroll
+    for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+      for (int qb = 0; qb < NQB; ++qb) s[kb][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < NKS; ++ks)
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+          s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][ks], qf[qb][ks], s[kb][qb], 0, 0, 0);
+    }
+    if (AHEAD && tile0 + tile_step <= last_q) load_keys(tile0 + tile_step);
     // the cap, the bias by distance, and -inf for what a query may not see
     const bool full_tile = tile0 + 63 <= first_q && tile0 >= lo_last;
 #pragma unroll
@@ -234,6 +275,7 @@ __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __re
 #pragma unroll
         for (int i = 0; i < 4; ++i) o[db][qb][i] *= alpha;
     }
+    if (!AHEAD) load_values(tile0);
 #pragma unroll
     for (int t = 0; t < 2; ++t) {
       if (tile0 + 32 * t > last_q) continue;
@@ -242,37 +284,14 @@ __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __re
       for (int qb = 0; qb < NQB; ++qb)
 #pragma unroll
         for (int j = 0; j < 8; ++j) pb[qb][j] = (bf16_t)s[2 * t + (j >> 2)][qb][j & 3];
-      const bf16_t* vbase[2];
-      bool vok[2];
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const int key0 = tile0 + 32 * t + 16 * b;
-        int page = -1;
-        if (key0 <= last_q) page = tab[key0 / page_size];
-        vok[b] = page >= 0 && page < num_pages;
-        vbase[b] = v_pages + (size_t)(vok[b] ? page : 0) * page_stride + (size_t)kvh * head_size * page_size +
-                   key0 % page_size + 4 * g;
-      }
-      const bool tail = tile0 + 32 * t + 32 > total;   // some keys of this step lie beyond the request
 #pragma unroll
       for (int db = 0; db < NDB; ++db) {
         if (db >= ndb) continue;
-        const int d = 16 * db + r;
-        bf16x8 vf;
+        bf16x8 v8;
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          bf16x4 v4 = {0, 0, 0, 0};
-          if (vok[b]) v4 = *(const bf16x4*)(vbase[b] + (size_t)d * page_size);
-          if (tail) {
+        for (int j = 0; j < 8; ++j) v8[j] = vf[db][2 * t + (j >> 2)][j & 3];
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (tile0 + 32 * t + 16 * b + 4 * g + i >= total) v4[i] = 0;
-          }
-#pragma unroll
-          for (int i = 0; i < 4; ++i) vf[4 * b + i] = v4[i];
-        }
-#pragma unroll
-        for (int qb = 0; qb < NQB; ++qb) o[db][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb[qb], o[db][qb], 0, 0, 0);
+        for (int qb = 0; qb < NQB; ++qb) o[db][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(v8, pb[qb], o[db][qb], 0, 0, 0);
       }
     }
   }
