@@ -444,6 +444,8 @@ def main():
                     help="instead: this design at sizes of published layers beside the closest design the engine had, "
                          "at equal sizes (--layers of them, 4 by default): decode and prompt throughput and every "
                          "kernel's rates; prints its own line")
+    ap.add_argument("--beside-alone", default=None, metavar="SIZE",
+                    help="with --beside: the new design alone at this one size (\"2048 wide\"), for profiles")
     args = ap.parse_args()
     if args.beside:
         return beside(args)
@@ -575,10 +577,12 @@ def beside(args):
            "unit": "tokens/s", "dtype": args.dtype, "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
            "data": "synthetic (seeded random weights and token ids)", "layers": layers, "context": context, "sizes": {}}
     for size, (make, preset) in BESIDE[args.beside].items():
+        if args.beside_alone and size != args.beside_alone:
+            continue
         row = {}
         other = (preset[0], preset[1](layers)) if isinstance(preset, tuple) else (
             "opt", dict(PRESETS[preset], num_hidden_layers=layers, max_position_embeddings=max(2048, context)))
-        for design, raw in ((args.beside, make(layers)), other):
+        for design, raw in ((args.beside, make(layers)),) + (() if args.beside_alone else (other,)):
             bench = Bench(raw, args.dtype, args.batch, context, step_tokens=tokens)
             keep_busy(bench.runner.ops, torch, 1.0)
             value, sec, read = bench.decode(args.batch, args.steps, args.warmup)

@@ -226,6 +226,9 @@ def _standout(dtype, case, seed):
     dict(h=6, g=2, n=48, v=80, chunk=70, length=390, run=200, ps=64, back=40, rows=16, far=70, scale=0.5, cap=25.0),
     dict(h=8, g=2, n=96, v=64, chunk=256, length=1000, run=300, ps=64, back=231, rows=16, far=256, scale=0.3, cap=30.0),  # a long portion over a chunk's edge
     dict(h=8, g=2, n=96, v=64, chunk=256, length=1000, run=300, ps=64, back=232, rows=16, far=256, scale=0.3, cap=30.0),
+    dict(h=4, g=2, n=32, v=32, chunk=100, length=330, run=130, ps=48, back=29, rows=8, far=100, scale=0.8, cap=30.0),    # pages that are no power of two
+    dict(h=4, g=2, n=32, v=32, chunk=100, length=330, run=130, ps=48, back=30, rows=8, far=100, scale=0.8, cap=30.0),
+    dict(h=2, g=1, n=64, v=64, chunk=None, length=600, run=200, ps=64, back=500, rows=32, far=5000, scale=0.4, cap=None),  # a long bias table
 ])
 @pytest.mark.parametrize("one_wave_a_query", [False, True])
 def test_scored_attention_finds_the_key_that_stands_out(name, dtype, tol, case, one_wave_a_query):

@@ -538,14 +538,41 @@ struct PrefillTileLayout {
   static constexpr int VSTR = FAST ? 64 + 16 : 64 + 8;          // per staged value row (one element, 64 keys)
   static constexpr int KBUF = 64 * KSTR, VBUF = DMAX * VSTR;
 };
-template <int NDB, bool FAST, int GROUPS>
+// What changes the scores, the mask and the result of the staged kernel (SCORED): a cap c on the scores
+// (c tanh(s / c)), a bias by the distance between query and key (`[heads, far + 1]` float32, read at
+// min(i - j, far); staged in LDS behind the tiles where `bias_in_lds`), visibility inside chunks of the request,
+// a gate on the result (the first `value_size` elements of a head times sigmoid(gate)), a factor on the result,
+// and result rows that lie `out_ld` elements apart.
+struct ScoreMods {
+  float softcap;
+  const float* bias;
+  int far, bias_in_lds;
+  int chunk;
+  const float* gate;
+  long long gate_ld, out_ld;
+  float out_scale;
+  int value_size, vector_store;
+};
+
+__device__ __forceinline__ int first_visible_key(int pos, int window, int chunk) {
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos - pos % chunk);
+  return lo;
+}
+
+// tanh from one exponential and one reciprocal: 1 - 2 / (1 + e^(2x)); +-1 where the exponential leaves the range.
+__device__ __forceinline__ float tanh_by_exp(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * (2.f * LOG2E)));
+}
+
+template <int NDB, bool FAST, int GROUPS, bool SCORED = false>
 __global__ void __launch_bounds__(256 * GROUPS, (NDB <= 8 && GROUPS == 1 ? 2 : 1))
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
                              const int* __restrict__ cached_lens, const int* __restrict__ table, int table_width,
                              int page_shift, int num_pages, const int* __restrict__ tile_run,
                              const int* __restrict__ tile_q0, bf16_t* __restrict__ out, int num_heads, int num_kv,
-                             int head_size, int window, int page_pad) {
+                             int head_size, int window, int page_pad, ScoreMods sm) {
   constexpr int NKS = (NDB + 1) / 2;
   constexpr int DMAX = 16 * NDB;
   using Layout = PrefillTileLayout<NDB, FAST>;
@@ -593,10 +620,20 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   }
   // block-wide range of key tiles; each wave computes only the tiles its own queries can see
   const int blk_last = cached + min(q0 + PREFILL_Q_TILE - 1, qlen - 1);
-  const int blk_lo = window > 0 ? max(0, cached + q0 - window + 1) : 0;
+  const int chunk = SCORED ? sm.chunk : 0;
+  const int blk_lo = first_visible_key(cached + q0, window, chunk);
   const int last_q = cached + min(qw0 + 31, qlen - 1);
   const int first_q = cached + qw0;
-  const int lo = window > 0 ? max(0, first_q - window + 1) : 0;
+  const int lo = first_visible_key(first_q, window, chunk);
+  const int lo_last = first_visible_key(last_q, window, chunk);      // SCORED: tiles from here on need no lower mask
+  const int qlo[2] = {first_visible_key(qpos[0], window, chunk), first_visible_key(qpos[1], window, chunk)};
+  const float* bias_glob = nullptr;
+  float* bias_lds = (float*)(smem + GROUPS * 2 * (KBUF + VBUF));
+  if (SCORED && sm.bias) {
+    bias_glob = sm.bias + (size_t)h * (sm.far + 1);
+    if (sm.bias_in_lds)      // read after the first barrier of the loop over tiles
+      for (int i = threadIdx.x; i <= sm.far; i += 256 * GROUPS) bias_lds[i] = bias_glob[i];
+  }
 
   float m[2] = {-INFINITY, -INFINITY}, l[2] = {0.f, 0.f};
   f32x4 o[NDB][2];
@@ -759,7 +796,31 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
       s[kb][1] = a1;
       if (KA == 2) __builtin_amdgcn_sched_barrier(0);
     }
-    const bool full_tile = tile0 + 63 <= first_q && (window <= 0 || tile0 > last_q - window);
+    const bool full_tile = SCORED ? tile0 + 63 <= first_q && tile0 >= lo_last
+                                  : tile0 + 63 <= first_q && (window <= 0 || tile0 > last_q - window);
+    if (SCORED) {
+      // the cap, then the bias by distance
+      const float cap = sm.softcap, inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+      auto modify = [&](auto bias_at) {
+#pragma unroll
+        for (int kb = 0; kb < 4; ++kb)
+#pragma unroll
+          for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              const int key = FAST ? tile0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + i : tile0 + 16 * kb + 4 * g + i;
+              float x = s[kb][qb][i];
+              if (cap > 0.f) x = cap * tanh_by_exp(x * inv_cap);
+              s[kb][qb][i] = x + bias_at(min(max(qpos[qb] - key, 0), sm.far));
+            }
+      };
+      if (!bias_glob)
+        modify([](int) { return 0.f; });
+      else if (sm.bias_in_lds)
+        modify([&](int i) { return bias_lds[i]; });
+      else
+        modify([&](int i) { return bias_glob[i]; });
+    }
     if (!full_tile) {
 #pragma unroll
       for (int kb = 0; kb < 4; ++kb)
@@ -768,7 +829,8 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
           for (int i = 0; i < 4; ++i) {
             const int key = FAST ? tile0 + 32 * (kb >> 1) + 8 * g + 4 * (kb & 1) + i : tile0 + 16 * kb + 4 * g + i;
-            const bool ok = key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
+            const bool ok = SCORED ? key <= qpos[qb] && key >= qlo[qb]
+                                   : key <= qpos[qb] && (window <= 0 || key > qpos[qb] - window);
             if (!ok) s[kb][qb][i] = -INFINITY;
           }
     }
@@ -882,6 +944,30 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   for (int qb = 0; qb < 2; ++qb) {
     const int qi = qw0 + 16 * qb + r;
     if (qi >= qlen) continue;
+    if (SCORED) {
+      const float inv = sm.out_scale / l[qb];
+      bf16_t* orow = out + (size_t)(t0 + qi) * sm.out_ld + h * head_size;
+      const float* gate = sm.gate ? sm.gate + (size_t)(t0 + qi) * sm.gate_ld + (size_t)h * sm.value_size : nullptr;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        if (db >= ndb) continue;
+        const int d0 = 16 * db + 4 * g;
+        bf16x4 v4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float x = o[db][qb][i] * inv;
+          if (gate && d0 + i < sm.value_size) x *= __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gate[d0 + i] * LOG2E));
+          v4[i] = (bf16_t)x;
+        }
+        if (sm.vector_store) {
+          *(bf16x4*)(orow + d0) = v4;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) orow[d0 + i] = v4[i];
+        }
+      }
+      continue;
+    }
     const float inv = 1.f / l[qb];
     bf16_t* orow = out + (size_t)(t0 + qi) * nq + h * head_size;
 #pragma unroll
@@ -895,32 +981,40 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   }
 }
 
-template <int NDB, bool FAST, int GROUPS>
+template <int NDB, bool FAST, int GROUPS, bool SCORED = false>
 static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
                               const bf16_t* v_pages, const int* run_start, const int* cached_lens, const int* table,
                               int table_width, int page_shift, int num_pages, const int* tile_run,
                               const int* tile_q0, bf16_t* out, int num_heads, int num_kv, int head_size,
-                              int window, int page_pad) {
+                              int window, int page_pad, ScoreMods sm = ScoreMods{}) {
   constexpr int DMAX = 16 * NDB;
   using Layout = PrefillTileLayout<NDB, FAST>;
-  constexpr size_t bytes = GROUPS * 2 * (size_t)(Layout::KBUF + Layout::VBUF) * sizeof(bf16_t);
-  static_assert(bytes <= 160 * 1024, "the staging buffers must fit the 160 KB of LDS");
-  static_assert(GROUPS == 1 || bytes >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
+  constexpr size_t tiles = GROUPS * 2 * (size_t)(Layout::KBUF + Layout::VBUF) * sizeof(bf16_t);
+  constexpr size_t limit = 160 * 1024;
+  size_t bytes = tiles;
+  if (SCORED) {
+    // the head's bias row lies behind the tiles where LDS has the room
+    const size_t row = sm.bias ? (size_t)(sm.far + 1) * sizeof(float) : 0;
+    sm.bias_in_lds = sm.bias && tiles + row <= limit;
+    if (sm.bias_in_lds) bytes += row;
+  }
+  static_assert(tiles <= limit, "the staging buffers must fit the 160 KB of LDS");
+  static_assert(GROUPS == 1 || tiles >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
                 "the partial results of the second set of waves must fit the staging buffers");
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST, GROUPS>,
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+    const size_t most = SCORED ? limit : tiles;
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST, GROUPS, SCORED>,
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);
     if (e != hipSuccess) {
-      tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
+      tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", most, hipGetErrorString(e));
       return 2;
     }
     configured = true;
   }
-  attention_prefill_lds_kernel<NDB, FAST, GROUPS><<<grid, 256 * GROUPS, bytes, stream>>>(q, k_pages, v_pages, run_start, cached_lens, table,
-                                                                 table_width, page_shift, num_pages, tile_run,
-                                                                 tile_q0, out, num_heads, num_kv, head_size, window,
-                                                                 page_pad);
+  attention_prefill_lds_kernel<NDB, FAST, GROUPS, SCORED><<<grid, 256 * GROUPS, bytes, stream>>>(
+      q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run, tile_q0, out,
+      num_heads, num_kv, head_size, window, page_pad, sm);
   return 0;
 }
 
@@ -1517,6 +1611,64 @@ extern "C" int tnx_attention_prefill(const void* q, const void* k_pages, const v
     LAUNCH_PREFILL(16);
 #undef LAUNCH_PREFILL
   TNX_CHECK_LAUNCH("attention_prefill");
+  return 0;
+}
+
+// The staged prompt kernel with what changes the scores, the mask and the result (see `ScoreMods`). Pages of a
+// power of two of keys. `sets`: 2, two sets of waves a block where LDS holds the buffers of both; 1, one.
+extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, const void* v_pages, const int* run_start,
+                                            const int* cached_lens, const int* table, int table_width, int page_size,
+                                            int num_pages, const int* tile_run, const int* tile_q0, int num_tiles,
+                                            int query_tile, void* out, long long out_ld, float out_scale,
+                                            const float* gate, long long gate_ld, const float* bias, int far,
+                                            float softcap, int window, int chunk, int num_heads, int num_kv,
+                                            int head_size, int value_size, int sets, int page_pad, hipStream_t stream) {
+  TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention_prefill_scored: bad distance between pages");
+  TNX_REQUIRE(query_tile == PREFILL_Q_TILE, "attention_prefill_scored: tiles of %d queries, the kernels take %d",
+              query_tile, PREFILL_Q_TILE);
+  TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_prefill_scored: bad head counts");
+  TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
+              "attention_prefill_scored: head size %d is not a multiple of 16 in [16, 256]", head_size);
+  TNX_REQUIRE(value_size > 0 && value_size <= head_size, "attention_prefill_scored: values of %d in heads of %d",
+              value_size, head_size);
+  TNX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
+              "attention_prefill_scored: page size %d is not a power of two from 16 on", page_size);
+  TNX_REQUIRE(out_ld >= (long long)num_heads * head_size, "attention_prefill_scored: result rows of %lld elements", out_ld);
+  TNX_REQUIRE(!gate || gate_ld >= (long long)num_heads * value_size, "attention_prefill_scored: gate rows of %lld elements", gate_ld);
+  TNX_REQUIRE(!bias || far >= 0, "attention_prefill_scored: a bias table needs its last distance");
+  TNX_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attention_prefill_scored: bad window, chunk or cap");
+  if (num_tiles <= 0) return 0;
+  TNX_REQUIRE((long long)num_tiles * num_heads < (1ll << 31), "attention_prefill_scored: too many tiles");
+  dim3 grid((unsigned)num_tiles * num_heads);
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  ScoreMods sm{softcap, bias, far, 0, chunk, gate, gate_ld, out_ld, out_scale, value_size,
+               out_ld % 4 == 0 && ((uintptr_t)out & 7) == 0};
+  int rc = -1;
+#define SCORED_ARGS                                                                                              \
+  grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, \
+      table_width, page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window, \
+      page_pad, sm
+#define LAUNCH_SCORED(NDB)                                                                                           \
+  {                                                                                                                  \
+    constexpr int G = NDB <= 8 ? 2 : 1;                                                                              \
+    const bool fast = NDB <= 8 && page_size >= 64 && head_size == 16 * NDB;                                          \
+    if (sets == 1)                                                                                                   \
+      rc = fast ? launch_prefill_lds<NDB, true, 1, true>(SCORED_ARGS) : launch_prefill_lds<NDB, false, 1, true>(SCORED_ARGS); \
+    else                                                                                                             \
+      rc = fast ? launch_prefill_lds<NDB, true, G, true>(SCORED_ARGS) : launch_prefill_lds<NDB, false, G, true>(SCORED_ARGS); \
+  }
+  if (head_size <= 64) {
+    LAUNCH_SCORED(4);
+  } else if (head_size <= 128) {
+    LAUNCH_SCORED(8);
+  } else {
+    LAUNCH_SCORED(16);
+  }
+#undef LAUNCH_SCORED
+#undef SCORED_ARGS
+  if (rc) return rc;
+  TNX_CHECK_LAUNCH("attention_prefill_scored");
   return 0;
 }
 

@@ -2,9 +2,13 @@
 //   min_gru                  S <- (1 - z) S + z c, the result S silu(g)
 //   channel_conv             a causal convolution of a few taps on every channel, with a bias and per-request state
 //   gated_linear_recurrence  S <- a S + sqrt(1 - a^2) i u with a = exp(rate sigmoid(r')), the result S gelu_tanh(y)
-// Gates, decays and state are float32 with full-precision exponentials. A thread owns one channel of one run and
-// walks its tokens; what does not depend on the state (loads, gates) is made eight tokens at a time ahead of the
-// chain. State lies by position: the token at position p reads place (p - 1) & 1 of two and writes place p & 1, so
+// Gates, decays and state are float32 with full-precision exponentials. In a step of single tokens a thread owns
+// one channel of one run; what does not depend on the state (loads, gates) is made eight tokens at a time ahead of
+// the chain. In a step with longer runs a run's tokens are cut into SEGMENTS parts that sixteen waves walk side by
+// side (`*_by_segments`): both recurrences are S <- a S + b, so a part taken from S = 0 leaves (A, B) = (the product
+// of its a, its last S), the parts' (A, B) meet in LDS, each part works out the S it begins with from those before
+// it (S <- A S + B), and walks its tokens again from there, now writing. A token's S is made by the same chain of
+// operations as by one thread alone from its part's first S on. State lies by position: the token at position p reads place (p - 1) & 1 of two and writes place p & 1, so
 // a step of single tokens that is recorded and run again reads what it read the first time.
 #include "common.h"
 
@@ -156,6 +160,123 @@ __global__ void __launch_bounds__(256) gated_linear_recurrence_kernel(Recurrence
   mine[(size_t)((p0 + n - 1) & 1) * a.channels + c] = s;
 }
 
+// ------------------------------------------------------------------------------------------ runs cut into parts
+
+constexpr int SEGMENTS = 16;          // waves a block: one part of the run each, 64 channels side by side
+constexpr int SEG_MIN = 4;            // tokens a part at least: shorter runs use fewer parts
+
+// What a recurrence S <- a S + b with a result S * f needs of a token: `Gate::ab(t, a, b)`, `Gate::factor(t)`.
+struct MinGruGate {
+  const float* proj;
+  int ld, inner, c;
+  float out_scale;
+  __device__ __forceinline__ void ab(size_t t, float& a, float& b) const {
+    const float* row = proj + t * ld;
+    const float z = sigmoid_full(row[c]);
+    const float u = row[inner + c];
+    const float cand = u >= 0.f ? u + 0.5f : sigmoid_full(u);
+    a = 1.f - z;
+    b = z * cand;
+  }
+  __device__ __forceinline__ float factor(size_t t) const {
+    const float g = proj[t * ld + 2 * inner + c];
+    return g * sigmoid_full(g) * out_scale;
+  }
+};
+
+struct LinearGate {
+  const float* gates;
+  const float* u;
+  const float* y;
+  long long y_ld;
+  size_t gates_ld;
+  int channels, c, at_r, at_i;
+  float bias_r, bias_i, rate, out_scale;
+  __device__ __forceinline__ void ab(size_t t, float& a, float& b) const {
+    const float log_a = rate * sigmoid_full(gates[t * gates_ld + at_r] + bias_r);
+    a = expf(log_a);
+    b = sqrtf(-expm1f(2.f * log_a)) * sigmoid_full(gates[t * gates_ld + at_i] + bias_i) * u[t * channels + c];
+  }
+  __device__ __forceinline__ float factor(size_t t) const {
+    return apply_act(y[t * y_ld + c], TNX_ACT_GELU_NEW) * out_scale;
+  }
+};
+
+// Tokens [from, to) of the step from state `s`; `prod` gathers the product of the a. WRITE: the results go out.
+template <bool WRITE, typename T, typename Gate>
+__device__ __forceinline__ void walk_part(const Gate& gate, int from, int to, float& s, float& prod, T* out,
+                                          long long out_ld, int c) {
+  for (int i0 = from; i0 < to; i0 += AHEAD) {
+    float a[AHEAD], b[AHEAD], f[AHEAD];
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= to) break;
+      gate.ab((size_t)(i0 + k), a[k], b[k]);
+      if (WRITE) f[k] = gate.factor((size_t)(i0 + k));
+    }
+#pragma unroll
+    for (int k = 0; k < AHEAD; ++k) {
+      if (i0 + k >= to) break;
+      s = a[k] * s + b[k];
+      if (WRITE)
+        out[(size_t)(i0 + k) * out_ld + c] = from_f32<T>(s * f[k]);
+      else
+        prod *= a[k];
+    }
+  }
+}
+
+// A block: 64 channels of one run, wave w the w-th part of its tokens. `carried` as above.
+template <typename T, typename Gate>
+__device__ __forceinline__ void recurrence_by_segments(const Gate& gate, bool live, int c, int channels, int first, int n,
+                                                       int p0, float* mine, T* out, long long out_ld) {
+  __shared__ float part_a[SEGMENTS][64], part_b[SEGMENTS][64];
+  const int lane = threadIdx.x & 63, seg = threadIdx.x >> 6;
+  const int parts = min(SEGMENTS, max(1, n / SEG_MIN));
+  const int len = (n + parts - 1) / parts;
+  const int from = first + min(n, seg * len), to = first + min(n, (seg + 1) * len);
+  const float s0 = live && p0 > 0 ? mine[(size_t)((p0 - 1) & 1) * channels + c] : 0.f;
+  float s = 0.f, prod = 1.f;
+  if (live && seg < parts - 1) walk_part<false, T>(gate, from, to, s, prod, out, out_ld, c);   // the last part's is not needed
+  part_a[seg][lane] = prod;
+  part_b[seg][lane] = s;
+  __syncthreads();
+  if (!live || from >= to) return;
+  s = s0;
+  for (int k = 0; k < seg; ++k) s = part_a[k][lane] * s + part_b[k][lane];
+  walk_part<true, T>(gate, from, to, s, prod, out, out_ld, c);
+  if (to == first + n) mine[(size_t)((p0 + n - 1) & 1) * channels + c] = s;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64 * SEGMENTS)
+min_gru_by_segments_kernel(const float* __restrict__ proj, int ld, int inner, const int* __restrict__ positions,
+                           const int* __restrict__ run_start, const int* __restrict__ slots, float* __restrict__ carried,
+                           T* __restrict__ out, long long out_ld, float out_scale) {
+  const int r = blockIdx.y, c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int first = run_start[r], n = run_start[r + 1] - first;
+  if (n <= 0) return;
+  const bool live = c < inner;
+  const MinGruGate gate{proj, ld, inner, live ? c : 0, out_scale};
+  recurrence_by_segments<T>(gate, live, c, inner, first, n, positions[first], carried + (size_t)slots[r] * 2 * inner, out,
+                            out_ld);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64 * SEGMENTS) gated_linear_recurrence_by_segments_kernel(RecurrenceArgs a) {
+  const int r = blockIdx.y, c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int first = a.run_start[r], n = a.run_start[r + 1] - first;
+  if (n <= 0) return;
+  const bool live = c < a.channels;
+  const int cc = live ? c : 0;
+  const int b = cc / a.w, j = cc - b * a.w;
+  const int at_r = b * 2 * a.w + j, at_i = at_r + a.w;
+  const LinearGate gate{a.gates, a.u, a.y, a.y_ld, (size_t)2 * a.channels, a.channels, cc, at_r, at_i,
+                        a.gate_bias[at_r], a.gate_bias[at_i], a.rate[cc], a.out_scale};
+  recurrence_by_segments<T>(gate, live, c, a.channels, first, n, a.positions[first],
+                            a.carried + (size_t)a.slots[r] * 2 * a.channels, (T*)a.out, a.out_ld);
+}
+
 }  // namespace
 
 extern "C" int tnx_min_gru(const float* proj, int ld, int inner, const int* positions, const int* run_start,
@@ -164,6 +285,17 @@ extern "C" int tnx_min_gru(const float* proj, int ld, int inner, const int* posi
   TNX_REQUIRE(tokens >= 0 && runs >= 0 && inner > 0 && ld >= 3 * inner && out_ld >= inner, "min_gru: bad sizes");
   TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "min_gru: dtype %d", out_dtype);
   if (tokens == 0 || runs == 0) return 0;
+  if (tokens > runs) {      // some run has several tokens
+    const dim3 by_parts((inner + 63) / 64, runs);
+    if (out_dtype == TNX_F32)
+      min_gru_by_segments_kernel<float><<<by_parts, 64 * SEGMENTS, 0, stream>>>(proj, ld, inner, positions, run_start, slots,
+                                                                                carried, (float*)out, out_ld, out_scale);
+    else
+      min_gru_by_segments_kernel<bf16_t><<<by_parts, 64 * SEGMENTS, 0, stream>>>(proj, ld, inner, positions, run_start, slots,
+                                                                                 carried, (bf16_t*)out, out_ld, out_scale);
+    TNX_CHECK_LAUNCH("min_gru_by_segments");
+    return 0;
+  }
   const dim3 grid((inner + 255) / 256, runs);
   if (out_dtype == TNX_F32)
     min_gru_kernel<float><<<grid, 256, 0, stream>>>(proj, ld, inner, positions, run_start, slots, carried, (float*)out,
@@ -208,6 +340,15 @@ extern "C" int tnx_gated_linear_recurrence(const float* gates, const float* gate
   if (tokens == 0 || runs == 0) return 0;
   RecurrenceArgs a{gates, gate_bias, u, y, y_ld, rate, positions, run_start, slots, carried, out, out_ld, out_scale,
                    channels, w};
+  if (tokens > runs) {      // some run has several tokens
+    const dim3 by_parts((channels + 63) / 64, runs);
+    if (out_dtype == TNX_F32)
+      gated_linear_recurrence_by_segments_kernel<float><<<by_parts, 64 * SEGMENTS, 0, stream>>>(a);
+    else
+      gated_linear_recurrence_by_segments_kernel<bf16_t><<<by_parts, 64 * SEGMENTS, 0, stream>>>(a);
+    TNX_CHECK_LAUNCH("gated_linear_recurrence_by_segments");
+    return 0;
+  }
   const dim3 grid((channels + 255) / 256, runs);
   if (out_dtype == TNX_F32)
     gated_linear_recurrence_kernel<float><<<grid, 256, 0, stream>>>(a);

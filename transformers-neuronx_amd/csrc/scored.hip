@@ -336,6 +336,7 @@ attention_scored_tiles_kernel(ScoredArgs a, const int* __restrict__ run_start, c
   const int t0 = run_start[run], qlen = run_start[run + 1] - t0, cached = cached_lens[run];
   const float* bias_row = a.bias ? a.bias + (size_t)h * (a.far + 1) : nullptr;
   if (bias_row && bias_in_lds) {
+#pragma unroll 4
     for (int i = threadIdx.x; i <= a.far; i += 256) lds[i] = bias_row[i];
     __syncthreads();
     bias_row = lds;
@@ -387,11 +388,13 @@ attention_scored_tiles_kernel(ScoredArgs a, const int* __restrict__ run_start, c
 }
 
 // A run of one token and one key/value head: column c is query head `kvh * pack + 16 * blockIdx.z + c` of the
-// `pack` that share the keys. Wave w takes the tiles w, w + 4, ...; waves 1 to 3 leave their maxima, sums and
-// weighted values (float32) in LDS and wave 0 joins them. Dynamic LDS: 3 * 16 * (16 NDB + 4) floats, then the
-// bias rows of the block's heads, where `bias_in_lds`.
+// `pack` that share the keys. Wave w of SINGLE_WAVES takes the tiles w, w + SINGLE_WAVES, ...; all but the first
+// leave their maxima, sums and weighted values (float32) in LDS and the first joins them. Dynamic LDS:
+// (SINGLE_WAVES - 1) * 16 * (16 NDB + 4) floats, then the bias rows of the block's heads, where `bias_in_lds`.
+constexpr int SINGLE_WAVES = 8;
+
 template <int NDB>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64 * SINGLE_WAVES)
 attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, const int* __restrict__ cached_lens,
                                const int* __restrict__ single_runs, int bias_in_lds, int vector_store) {
   extern __shared__ float lds[];
@@ -409,10 +412,11 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
   const int head = kvh * pack + col0 + min(r, cols - 1);
   const bool live = r < cols;
   const int token = run_start[run], pos = cached_lens[run];
-  float* bias_lds = lds + 3 * 16 * PART;
+  float* bias_lds = lds + (SINGLE_WAVES - 1) * 16 * PART;
   if (a.bias && bias_in_lds) {
     const float* rows = a.bias + (size_t)(kvh * pack + col0) * (a.far + 1);
-    for (int i = threadIdx.x; i < cols * (a.far + 1); i += 256) bias_lds[i] = rows[i];
+#pragma unroll 4
+    for (int i = threadIdx.x; i < cols * (a.far + 1); i += 64 * SINGLE_WAVES) bias_lds[i] = rows[i];
     __syncthreads();
   }
   const int nq = a.num_heads * head_size;
@@ -436,7 +440,7 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
 #pragma unroll
   for (int db = 0; db < NDB; ++db) o[db][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
   scored_walk<NDB, 1>(a, tab, page_stride, kvh, qf, qpos, qlo, bias, pos, pos, lo, pos + 1, (lo / 64) * 64 + 64 * wave,
-                      256, m, l, o);
+                      64 * SINGLE_WAVES, m, l, o);
   if (wave > 0) {
     float* part = lds + ((wave - 1) * 16 + r) * PART;
     if (g == 0) {
@@ -450,7 +454,7 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
   __syncthreads();
   if (wave > 0 || !live) return;
 #pragma unroll
-  for (int w = 0; w < 3; ++w) {
+  for (int w = 0; w < SINGLE_WAVES - 1; ++w) {
     const float* part = lds + (w * 16 + r) * PART;
     const float m2 = part[0], l2 = part[1];
     const float m_new = fmaxf(m[0], m2);
@@ -556,20 +560,31 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
   }
   if (num_single > 0) {
     const int ndb = head_size <= 64 ? 4 : head_size <= 128 ? 8 : 16;
-    const size_t parts = (size_t)3 * 16 * (16 * ndb + 4) * sizeof(float);
+    const size_t parts = (size_t)(SINGLE_WAVES - 1) * 16 * (16 * ndb + 4) * sizeof(float);
     const size_t rows = bias ? (size_t)(pack < 16 ? pack : 16) * (far + 1) * sizeof(float) : 0;
-    const int in_lds = bias && parts + rows <= budget;
+    const size_t most = 160 * 1024;
+    const int in_lds = bias && parts + rows <= most;
     const size_t lds = parts + (in_lds ? rows : 0);
     dim3 grid((unsigned)num_single, (unsigned)num_kv, (unsigned)((pack + 15) / 16));
-#define LAUNCH_SINGLE(NDB)                                                                                          \
-  attention_scored_single_kernel<NDB><<<grid, 256, lds, stream>>>(a, run_start, cached_lens, single_runs, in_lds, \
-                                                                  vector_store)
-    if (ndb == 4)
-      LAUNCH_SINGLE(4);
-    else if (ndb == 8)
-      LAUNCH_SINGLE(8);
-    else
-      LAUNCH_SINGLE(16);
+#define LAUNCH_SINGLE(NDB)                                                                                       \
+  {                                                                                                              \
+    static bool configured = false;                                                                              \
+    if (!configured) {                                                                                           \
+      hipError_t e = hipFuncSetAttribute((const void*)attention_scored_single_kernel<NDB>,                       \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);                 \
+      TNX_REQUIRE(e == hipSuccess, "attention_scored_single: cannot reserve LDS: %s", hipGetErrorString(e));     \
+      configured = true;                                                                                         \
+    }                                                                                                            \
+    attention_scored_single_kernel<NDB><<<grid, 64 * SINGLE_WAVES, lds, stream>>>(a, run_start, cached_lens,     \
+                                                                                   single_runs, in_lds, vector_store); \
+  }
+    if (ndb == 4) {
+      LAUNCH_SINGLE(4)
+    } else if (ndb == 8) {
+      LAUNCH_SINGLE(8)
+    } else {
+      LAUNCH_SINGLE(16)
+    }
 #undef LAUNCH_SINGLE
     TNX_CHECK_LAUNCH("attention_scored_single");
   }

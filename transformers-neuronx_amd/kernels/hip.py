@@ -61,6 +61,10 @@ _SIGNATURES = {
                           _c_void_p],
         "tnx_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                               _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+        "tnx_attention_prefill_scored": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                                         _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_ll, _c_float,
+                                         _c_void_p, _c_ll, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
+                                         _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                   _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                                   _c_int, _c_int, _c_int, _c_void_p],
@@ -1520,14 +1524,25 @@ class HipOps:
         work = (self._scored_work(ctx, num_heads, num_kv_heads, head_size, window, chunk, q.element_size())
                 if debug.timer() is not None else None)
         if self.dtype == torch.bfloat16 and not self.force_plain_attention and "tile_run" in ctx.plan:
-            # on the matrix unit: the runs of several tokens by tiles of queries, the runs of one token by key/value head
+            # on the matrix unit: the runs of several tokens by tiles of queries (through LDS where the pages are a
+            # power of two of keys), the runs of one token by key/value head
             tiles, single = ctx.plan["tile_run"], ctx.plan["decode_runs"]
-            self._call("scored", "tnx_attention_scored_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.run_start),
-                       _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size, num_pages, _ptr(tiles),
-                       _ptr(ctx.plan["tile_start"]), tiles.numel(), QUERY_TILE, _ptr(single), single.numel(), _ptr(out),
-                       out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far, float(softcap or 0.0),
-                       int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size, value_size, pad, _stream(),
-                       work=work)
+            staged = tiles.numel() > 0 and view.page_size & (view.page_size - 1) == 0
+            if staged:
+                sets = 1 if (int(self.prefill_direct) or self._prefill_sets(ctx, num_heads, int(window or chunk or 0))) == 2 else 2
+                self._call("attention", "tnx_attention_prefill_scored", _ptr(q), _ptr(k_pages), _ptr(v_pages),
+                           _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size,
+                           num_pages, _ptr(tiles), _ptr(ctx.plan["tile_start"]), tiles.numel(), QUERY_TILE, _ptr(out), out_ld,
+                           float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far, float(softcap or 0.0),
+                           int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size, value_size, sets, pad,
+                           _stream(), work=work)
+            if not staged or single.numel():
+                self._call("scored", "tnx_attention_scored_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.run_start),
+                           _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size, num_pages, _ptr(tiles),
+                           _ptr(ctx.plan["tile_start"]), 0 if staged else tiles.numel(), QUERY_TILE, _ptr(single),
+                           single.numel(), _ptr(out), out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far,
+                           float(softcap or 0.0), int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size,
+                           value_size, pad, _stream(), work=None if staged else work)
             return out
         self._call("scored", "tnx_attention_scored", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
