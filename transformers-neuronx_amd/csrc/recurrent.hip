@@ -4,7 +4,7 @@
 //   gated_linear_recurrence  S <- a S + sqrt(1 - a^2) i u with a = exp(rate sigmoid(r')), the result S gelu_tanh(y)
 // Gates, decays and state are float32 with full-precision exponentials. In a step of single tokens a thread owns
 // one channel of one run; what does not depend on the state (loads, gates) is made eight tokens at a time ahead of
-// the chain. In a step with longer runs a run's tokens are cut into SEGMENTS parts that sixteen waves walk side by
+// the chain. In a step with longer runs a run's tokens are cut into parts that a block's sixteen waves walk side by
 // side (`*_by_segments`): both recurrences are S <- a S + b, so a part taken from S = 0 leaves (A, B) = (the product
 // of its a, its last S), the parts' (A, B) meet in LDS, each part works out the S it begins with from those before
 // it (S <- A S + B), and walks its tokens again from there, now writing. A token's S is made by the same chain of
@@ -162,8 +162,10 @@ __global__ void __launch_bounds__(256) gated_linear_recurrence_kernel(Recurrence
 
 // ------------------------------------------------------------------------------------------ runs cut into parts
 
-constexpr int SEGMENTS = 16;          // waves a block: one part of the run each, 64 channels side by side
+constexpr int SEGMENTS = 16;          // waves a block
 constexpr int SEG_MIN = 4;            // tokens a part at least: shorter runs use fewer parts
+// A block takes CH = 16 channels of a run and cuts its tokens into 1024 / CH = 64 parts, four a wave (a lane's
+// neighbours in memory are 16 channels, 64 bytes): 2,048 channels of one prompt make 128 blocks.
 
 // What a recurrence S <- a S + b with a result S * f needs of a token: `Gate::ab(t, a, b)`, `Gate::factor(t)`.
 struct MinGruGate {
@@ -227,12 +229,13 @@ __device__ __forceinline__ void walk_part(const Gate& gate, int from, int to, fl
 }
 
 // A block: 64 channels of one run, wave w the w-th part of its tokens. `carried` as above.
-template <typename T, typename Gate>
+template <int CH, typename T, typename Gate>
 __device__ __forceinline__ void recurrence_by_segments(const Gate& gate, bool live, int c, int channels, int first, int n,
                                                        int p0, float* mine, T* out, long long out_ld) {
-  __shared__ float part_a[SEGMENTS][64], part_b[SEGMENTS][64];
-  const int lane = threadIdx.x & 63, seg = threadIdx.x >> 6;
-  const int parts = min(SEGMENTS, max(1, n / SEG_MIN));
+  constexpr int NSEG = 64 * SEGMENTS / CH;
+  __shared__ float part_a[NSEG][CH], part_b[NSEG][CH];
+  const int lane = threadIdx.x % CH, seg = threadIdx.x / CH;
+  const int parts = min(NSEG, max(1, n / SEG_MIN));
   const int len = (n + parts - 1) / parts;
   const int from = first + min(n, seg * len), to = first + min(n, (seg + 1) * len);
   const float s0 = live && p0 > 0 ? mine[(size_t)((p0 - 1) & 1) * channels + c] : 0.f;
@@ -248,23 +251,23 @@ __device__ __forceinline__ void recurrence_by_segments(const Gate& gate, bool li
   if (to == first + n) mine[(size_t)((p0 + n - 1) & 1) * channels + c] = s;
 }
 
-template <typename T>
+template <int CH, typename T>
 __global__ void __launch_bounds__(64 * SEGMENTS)
 min_gru_by_segments_kernel(const float* __restrict__ proj, int ld, int inner, const int* __restrict__ positions,
                            const int* __restrict__ run_start, const int* __restrict__ slots, float* __restrict__ carried,
                            T* __restrict__ out, long long out_ld, float out_scale) {
-  const int r = blockIdx.y, c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int r = blockIdx.y, c = blockIdx.x * CH + threadIdx.x % CH;
   const int first = run_start[r], n = run_start[r + 1] - first;
   if (n <= 0) return;
   const bool live = c < inner;
   const MinGruGate gate{proj, ld, inner, live ? c : 0, out_scale};
-  recurrence_by_segments<T>(gate, live, c, inner, first, n, positions[first], carried + (size_t)slots[r] * 2 * inner, out,
+  recurrence_by_segments<CH, T>(gate, live, c, inner, first, n, positions[first], carried + (size_t)slots[r] * 2 * inner, out,
                             out_ld);
 }
 
-template <typename T>
+template <int CH, typename T>
 __global__ void __launch_bounds__(64 * SEGMENTS) gated_linear_recurrence_by_segments_kernel(RecurrenceArgs a) {
-  const int r = blockIdx.y, c = blockIdx.x * 64 + (threadIdx.x & 63);
+  const int r = blockIdx.y, c = blockIdx.x * CH + threadIdx.x % CH;
   const int first = a.run_start[r], n = a.run_start[r + 1] - first;
   if (n <= 0) return;
   const bool live = c < a.channels;
@@ -273,7 +276,7 @@ __global__ void __launch_bounds__(64 * SEGMENTS) gated_linear_recurrence_by_segm
   const int at_r = b * 2 * a.w + j, at_i = at_r + a.w;
   const LinearGate gate{a.gates, a.u, a.y, a.y_ld, (size_t)2 * a.channels, a.channels, cc, at_r, at_i,
                         a.gate_bias[at_r], a.gate_bias[at_i], a.rate[cc], a.out_scale};
-  recurrence_by_segments<T>(gate, live, c, a.channels, first, n, a.positions[first],
+  recurrence_by_segments<CH, T>(gate, live, c, a.channels, first, n, a.positions[first],
                             a.carried + (size_t)a.slots[r] * 2 * a.channels, (T*)a.out, a.out_ld);
 }
 
@@ -286,13 +289,16 @@ extern "C" int tnx_min_gru(const float* proj, int ld, int inner, const int* posi
   TNX_REQUIRE(out_dtype == TNX_F32 || out_dtype == TNX_BF16, "min_gru: dtype %d", out_dtype);
   if (tokens == 0 || runs == 0) return 0;
   if (tokens > runs) {      // some run has several tokens
-    const dim3 by_parts((inner + 63) / 64, runs);
-    if (out_dtype == TNX_F32)
-      min_gru_by_segments_kernel<float><<<by_parts, 64 * SEGMENTS, 0, stream>>>(proj, ld, inner, positions, run_start, slots,
-                                                                                carried, (float*)out, out_ld, out_scale);
-    else
-      min_gru_by_segments_kernel<bf16_t><<<by_parts, 64 * SEGMENTS, 0, stream>>>(proj, ld, inner, positions, run_start, slots,
-                                                                                 carried, (bf16_t*)out, out_ld, out_scale);
+    const dim3 by_parts((inner + 15) / 16, runs);
+#define LAUNCH_MIN_GRU(CH, T)                                                                                          \
+  min_gru_by_segments_kernel<CH, T><<<by_parts, 64 * SEGMENTS, 0, stream>>>(proj, ld, inner, positions, run_start, slots, \
+                                                                            carried, (T*)out, out_ld, out_scale)
+    if (out_dtype == TNX_F32) {
+      LAUNCH_MIN_GRU(16, float);
+    } else {
+      LAUNCH_MIN_GRU(16, bf16_t);
+    }
+#undef LAUNCH_MIN_GRU
     TNX_CHECK_LAUNCH("min_gru_by_segments");
     return 0;
   }
@@ -341,11 +347,11 @@ extern "C" int tnx_gated_linear_recurrence(const float* gates, const float* gate
   RecurrenceArgs a{gates, gate_bias, u, y, y_ld, rate, positions, run_start, slots, carried, out, out_ld, out_scale,
                    channels, w};
   if (tokens > runs) {      // some run has several tokens
-    const dim3 by_parts((channels + 63) / 64, runs);
+    const dim3 by_parts((channels + 15) / 16, runs);
     if (out_dtype == TNX_F32)
-      gated_linear_recurrence_by_segments_kernel<float><<<by_parts, 64 * SEGMENTS, 0, stream>>>(a);
+      gated_linear_recurrence_by_segments_kernel<16, float><<<by_parts, 64 * SEGMENTS, 0, stream>>>(a);
     else
-      gated_linear_recurrence_by_segments_kernel<bf16_t><<<by_parts, 64 * SEGMENTS, 0, stream>>>(a);
+      gated_linear_recurrence_by_segments_kernel<16, bf16_t><<<by_parts, 64 * SEGMENTS, 0, stream>>>(a);
     TNX_CHECK_LAUNCH("gated_linear_recurrence_by_segments");
     return 0;
   }
