@@ -387,8 +387,10 @@ attention_scored_tiles_kernel(ScoredArgs a, const int* __restrict__ run_start, c
   }
 }
 
-// A run of one token and one key/value head: column c is query head `kvh * pack + 16 * blockIdx.z + c` of the
-// `pack` that share the keys. Wave w of SINGLE_WAVES takes the tiles w, w + SINGLE_WAVES, ...; all but the first
+// A run of one token and one key/value head: column c is query head `kvh * pack + width * blockIdx.z + c` of the
+// `pack` that share the keys, `width` (up to 16) of them a block: all of them where the blocks are many, fewer
+// where a block a key/value head would leave most of the chip idle (the heads' blocks then read the same keys at
+// the same time, and all but the first find them in the cache). Wave w of SINGLE_WAVES takes the tiles w, w + SINGLE_WAVES, ...; all but the first
 // leave their maxima, sums and weighted values (float32) in LDS and the first joins them. Dynamic LDS:
 // (SINGLE_WAVES - 1) * 16 * (16 NDB + 4) floats, then the bias rows of the block's heads, where `bias_in_lds`.
 constexpr int SINGLE_WAVES = 8;
@@ -396,7 +398,7 @@ constexpr int SINGLE_WAVES = 8;
 template <int NDB>
 __global__ void __launch_bounds__(64 * SINGLE_WAVES)
 attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, const int* __restrict__ cached_lens,
-                               const int* __restrict__ single_runs, int bias_in_lds, int vector_store) {
+                               const int* __restrict__ single_runs, int width, int bias_in_lds, int vector_store) {
   extern __shared__ float lds[];
   constexpr int NKS = (NDB + 1) / 2;
   constexpr int PART = 16 * NDB + 4;      // maximum, sum, two unused, the values (16-byte rows)
@@ -407,8 +409,8 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
   const int r = lane & 15, g = lane >> 4;
   const int run = single_runs[blockIdx.x], kvh = blockIdx.y;
   const int pack = a.num_heads / a.num_kv;
-  const int col0 = 16 * blockIdx.z;
-  const int cols = min(16, pack - col0);
+  const int col0 = width * blockIdx.z;
+  const int cols = min(width, pack - col0);
   const int head = kvh * pack + col0 + min(r, cols - 1);
   const bool live = r < cols;
   const int token = run_start[run], pos = cached_lens[run];
@@ -561,11 +563,14 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
   if (num_single > 0) {
     const int ndb = head_size <= 64 ? 4 : head_size <= 128 ? 8 : 16;
     const size_t parts = (size_t)(SINGLE_WAVES - 1) * 16 * (16 * ndb + 4) * sizeof(float);
-    const size_t rows = bias ? (size_t)(pack < 16 ? pack : 16) * (far + 1) * sizeof(float) : 0;
+    // query heads a block: 16 (or all), halved while the blocks are fewer than the chip's compute units
+    int width = pack < 16 ? pack : 16;
+    while (width > 1 && (long long)num_single * num_kv * ((pack + width - 1) / width) < 256) width = (width + 1) / 2;
+    const size_t rows = bias ? (size_t)width * (far + 1) * sizeof(float) : 0;
     const size_t most = 160 * 1024;
     const int in_lds = bias && parts + rows <= most;
     const size_t lds = parts + (in_lds ? rows : 0);
-    dim3 grid((unsigned)num_single, (unsigned)num_kv, (unsigned)((pack + 15) / 16));
+    dim3 grid((unsigned)num_single, (unsigned)num_kv, (unsigned)((pack + width - 1) / width));
 #define LAUNCH_SINGLE(NDB)                                                                                       \
   {                                                                                                              \
     static bool configured = false;                                                                              \
@@ -576,7 +581,7 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
       configured = true;                                                                                         \
     }                                                                                                            \
     attention_scored_single_kernel<NDB><<<grid, 64 * SINGLE_WAVES, lds, stream>>>(a, run_start, cached_lens,     \
-                                                                                   single_runs, in_lds, vector_store); \
+                                                                                   single_runs, width, in_lds, vector_store); \
   }
     if (ndb == 4) {
       LAUNCH_SINGLE(4)
