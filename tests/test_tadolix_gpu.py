@@ -231,6 +231,9 @@ def _standout(dtype, case, seed):
     dict(h=4, g=2, n=32, v=32, chunk=100, length=330, run=130, ps=48, back=29, rows=8, far=100, scale=0.8, cap=30.0),    # pages that are no power of two
     dict(h=4, g=2, n=32, v=32, chunk=100, length=330, run=130, ps=48, back=30, rows=8, far=100, scale=0.8, cap=30.0),
     dict(h=2, g=1, n=64, v=64, chunk=None, length=600, run=200, ps=64, back=500, rows=32, far=5000, scale=0.4, cap=None),  # a long bias table
+    dict(h=4, g=2, n=160, v=144, chunk=90, length=300, run=140, ps=16, back=29, rows=12, far=90, scale=0.15, cap=35.0),   # heads beyond 128 elements
+    dict(h=4, g=2, n=160, v=144, chunk=90, length=300, run=1, ps=64, back=30, rows=12, far=90, scale=0.15, cap=35.0),
+    dict(h=3, g=1, n=200, v=256, chunk=None, length=200, run=1, ps=16, back=199, rows=8, far=300, scale=0.12, cap=None),
 ])
 @pytest.mark.parametrize("one_wave_a_query", [False, True])
 def test_scored_attention_finds_the_key_that_stands_out(name, dtype, tol, case, one_wave_a_query):
