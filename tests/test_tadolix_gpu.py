@@ -275,11 +275,12 @@ def test_scored_attention_finds_the_key_that_stands_out(name, dtype, tol, case, 
     _close(got.view(run, h, d)[:, :, :v].reshape(run, h * v), want, tol if dtype == torch.float32 else 4e-2)
 
 
-@pytest.mark.parametrize("pad", [0, 2, 3])
-def test_scored_attention_of_a_mixed_step_into_columns_of_a_wider_buffer(pad):
+@pytest.mark.parametrize("pad,splits", [(0, None), (2, 1), (3, 3), (0, 8)])
+def test_scored_attention_of_a_mixed_step_into_columns_of_a_wider_buffer(pad, splits):
     """Runs of one token (each key/value head's query heads side by side, 20 of them: two blocks of columns)
     beside a portion and a whole prompt in one step, written times a factor into a slice of a buffer whose rows
-    are not multiples of 8 bytes apart; against the general kernel, and the columns beside the slice untouched."""
+    are not multiples of 8 bytes apart, a decoded token's keys in one block or shared out over several (more
+    blocks than it has tiles among them); against the general kernel, and the columns beside the slice untouched."""
     from transformers_neuronx_amd.kernels.attention_plan import attention_plan
     from transformers_neuronx_amd.parts.mixer import bias_by_distance
     h, g, n, v, d, ps = 40, 2, 32, 24, 32, 16
@@ -298,6 +299,7 @@ def test_scored_attention_of_a_mixed_step_into_columns_of_a_wider_buffer(pad):
     for plain in (False, True):
         ops = _ops(torch.bfloat16)
         ops.force_plain_attention = plain
+        ops.scored_decode_splits = splits
         k_pages = torch.zeros(pages + 2, g, ps, d, dtype=torch.bfloat16, device=DEV)
         v_pages = torch.zeros(pages + 2, g, d, ps, dtype=torch.bfloat16, device=DEV)
         gen2 = torch.Generator().manual_seed(4)

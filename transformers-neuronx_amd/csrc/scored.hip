@@ -148,13 +148,14 @@ __device__ __forceinline__ int first_visible(int pos, int window, int chunk) {
 // that the accumulators (lane = column, four consecutive keys a register group) are at once the B operand of
 // O^T += V^T P^T. A column has its own position (`qpos`), first visible key (`qlo`) and bias row (`bias`, by
 // distance, in LDS or global memory): the columns are 32 queries of one head, or the heads of one query.
-// Tiles `tile_begin`, `tile_begin + tile_step`, ... up to `last_q`, the last position among the columns;
+// Tiles `tile_begin`, `tile_begin + tile_step`, ... up to the key `stop` (at most `last_q`, the last position among
+// the columns);
 // `first_q` the first and `lo_last` the first visible key of the last: a tile between them needs no mask.
 template <int NDB, int NQB>
 __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __restrict__ tab, size_t page_stride,
                                             int kvh, const bf16x8 (&qf)[NQB][(NDB + 1) / 2], const int (&qpos)[NQB],
                                             const int (&qlo)[NQB], const float* const (&bias)[NQB], int first_q,
-                                            int last_q, int lo_last, int total, int tile_begin, int tile_step,
+                                            int last_q, int stop, int lo_last, int total, int tile_begin, int tile_step,
                                             float (&m)[NQB], float (&l)[NQB], f32x4 (&o)[NDB][NQB]) {
   constexpr int NKS = (NDB + 1) / 2;
   const bf16_t* k_pages = (const bf16_t*)a.k_pages;
@@ -215,9 +216,9 @@ __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __re
   // scores are made and the next tile's keys as soon as they are: both arrive while the scores are capped,
   // biased and turned into weights.
   constexpr bool AHEAD = NDB <= 8;
-  if (AHEAD && tile_begin <= last_q) load_keys(tile_begin);
+  if (AHEAD && tile_begin <= stop) load_keys(tile_begin);
 
-  for (int tile0 = tile_begin; tile0 <= last_q; tile0 += tile_step) {
+  for (int tile0 = tile_begin; tile0 <= stop; tile0 += tile_step) {
     f32x4 s[4][NQB];
     if (!AHEAD) load_keys(tile0);
     if (AHEAD) load_values(tile0);
@@ -231,7 +232,7 @@ __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __re
         for (int qb = 0; qb < NQB; ++qb)
           s[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[kb][ks], qf[qb][ks], s[kb][qb], 0, 0, 0);
     }
-    if (AHEAD && tile0 + tile_step <= last_q) load_keys(tile0 + tile_step);
+    if (AHEAD && tile0 + tile_step <= stop) load_keys(tile0 + tile_step);
     // the cap, the bias by distance, and -inf for what a query may not see
     const bool full_tile = tile0 + 63 <= first_q && tile0 >= lo_last;
 #pragma unroll
@@ -372,7 +373,7 @@ attention_scored_tiles_kernel(ScoredArgs a, const int* __restrict__ run_start, c
   for (int db = 0; db < NDB; ++db)
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) o[db][qb] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  scored_walk<NDB, 2>(a, tab, page_stride, kvh, qf, qpos, qlo, bias, first_q, last_q,
+  scored_walk<NDB, 2>(a, tab, page_stride, kvh, qf, qpos, qlo, bias, first_q, last_q, last_q,
                       first_visible(last_q, a.window, a.chunk), total, (lo / 64) * 64, 64, m, l, o);
 #pragma unroll
   for (int qb = 0; qb < 2; ++qb) {
@@ -388,9 +389,8 @@ attention_scored_tiles_kernel(ScoredArgs a, const int* __restrict__ run_start, c
 }
 
 // A run of one token and one key/value head: column c is query head `kvh * pack + width * blockIdx.z + c` of the
-// `pack` that share the keys, `width` (up to 16) of them a block: all of them where the blocks are many, fewer
-// where a block a key/value head would leave most of the chip idle (the heads' blocks then read the same keys at
-// the same time, and all but the first find them in the cache). Wave w of SINGLE_WAVES takes the tiles w, w + SINGLE_WAVES, ...; all but the first
+// `pack` that share the keys, `width` (up to 16) of them a block. `splits` blocks share the request's key tiles
+// (a block's waves take its share's tiles in turn) and leave what they have in `partial`. Wave w of SINGLE_WAVES takes the tiles w, w + SINGLE_WAVES, ...; all but the first
 // leave their maxima, sums and weighted values (float32) in LDS and the first joins them. Dynamic LDS:
 // (SINGLE_WAVES - 1) * 16 * (16 NDB + 4) floats, then the bias rows of the block's heads, where `bias_in_lds`.
 constexpr int SINGLE_WAVES = 8;
@@ -398,7 +398,8 @@ constexpr int SINGLE_WAVES = 8;
 template <int NDB>
 __global__ void __launch_bounds__(64 * SINGLE_WAVES)
 attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, const int* __restrict__ cached_lens,
-                               const int* __restrict__ single_runs, int width, int bias_in_lds, int vector_store) {
+                               const int* __restrict__ single_runs, int width, int splits, float* __restrict__ partial,
+                               int bias_in_lds, int vector_store) {
   extern __shared__ float lds[];
   constexpr int NKS = (NDB + 1) / 2;
   constexpr int PART = 16 * NDB + 4;      // maximum, sum, two unused, the values (16-byte rows)
@@ -407,7 +408,8 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
   const size_t page_stride = (size_t)a.num_kv * a.page_size * head_size + a.page_pad;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
-  const int run = single_runs[blockIdx.x], kvh = blockIdx.y;
+  const int single = blockIdx.x / splits, split = blockIdx.x - single * splits;
+  const int run = single_runs[single], kvh = blockIdx.y;
   const int pack = a.num_heads / a.num_kv;
   const int col0 = width * blockIdx.z;
   const int cols = min(width, pack - col0);
@@ -441,7 +443,12 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
   f32x4 o[NDB][1];
 #pragma unroll
   for (int db = 0; db < NDB; ++db) o[db][0] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  scored_walk<NDB, 1>(a, tab, page_stride, kvh, qf, qpos, qlo, bias, pos, pos, lo, pos + 1, (lo / 64) * 64 + 64 * wave,
+  // this block's share of the request's key tiles
+  const int tile_lo = (lo / 64) * 64;
+  const int tiles = (pos - tile_lo) / 64 + 1, share = (tiles + splits - 1) / splits;
+  const int begin = tile_lo + 64 * split * share;
+  const int stop = min(pos, begin + 64 * share - 1);
+  scored_walk<NDB, 1>(a, tab, page_stride, kvh, qf, qpos, qlo, bias, pos, pos, stop, lo, pos + 1, begin + 64 * wave,
                       64 * SINGLE_WAVES, m, l, o);
   if (wave > 0) {
     float* part = lds + ((wave - 1) * 16 + r) * PART;
@@ -472,11 +479,52 @@ attention_scored_single_kernel(ScoredArgs a, const int* __restrict__ run_start, 
         for (int i = 0; i < 4; ++i) o[db][0][i] = o[db][0][i] * mine + o2[i] * other;
       }
   }
+  if (splits > 1) {       // the blocks of a request meet in `attention_scored_join_kernel`
+    float* mine = partial + (((size_t)single * a.num_heads + head) * splits + split) * (head_size + 4);
+    if (g == 0) {
+      mine[0] = m[0];
+      mine[1] = l[0];
+    }
+#pragma unroll
+    for (int db = 0; db < NDB; ++db)
+      if (db < ndb) *(f32x4*)(mine + 4 + 16 * db + 4 * g) = o[db][0];
+    return;
+  }
   const float inv = a.out_scale / l[0];
 #pragma unroll
   for (int db = 0; db < NDB; ++db) {
     if (db >= ndb) continue;
     store_four(a, token, head, 16 * db + 4 * g, o[db][0], inv, vector_store != 0);
+  }
+}
+
+// What the `splits` blocks of a decoded token's (request, head) left (maximum, sum, weighted values): joined,
+// times the factor, through the gate, to the result. A block of 64 threads a (token, head).
+__global__ void __launch_bounds__(64)
+attention_scored_join_kernel(ScoredArgs a, const int* __restrict__ run_start, const int* __restrict__ single_runs,
+                             int splits, const float* __restrict__ partial) {
+  const int single = blockIdx.x, head = blockIdx.y;
+  const int token = run_start[single_runs[single]];
+  const int stride = a.head_size + 4;
+  const float* mine = partial + ((size_t)single * a.num_heads + head) * splits * stride;
+  float mm = -INFINITY;
+  for (int s = 0; s < splits; ++s) mm = fmaxf(mm, mine[s * stride]);
+  float ll = 0.f;
+  for (int s = 0; s < splits; ++s) {
+    const float ms = mine[s * stride];
+    ll += ms == -INFINITY ? 0.f : mine[s * stride + 1] * __expf(ms - mm);
+  }
+  bf16_t* orow = (bf16_t*)a.out + (size_t)token * a.out_ld + (size_t)head * a.head_size;
+  const float* gate = a.gate ? a.gate + (size_t)token * a.gate_ld + (size_t)head * a.value_size : nullptr;
+  for (int d = threadIdx.x; d < a.head_size; d += 64) {
+    float oo = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      const float ms = mine[s * stride];
+      if (ms != -INFINITY) oo += mine[s * stride + 4 + d] * __expf(ms - mm);
+    }
+    float x = oo * a.out_scale / ll;
+    if (gate && d < a.value_size) x *= 1.f / (1.f + __expf(-gate[d]));
+    orow[d] = (bf16_t)x;
   }
 }
 
@@ -523,8 +571,10 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
                                          long long out_ld, float out_scale, const float* gate, long long gate_ld,
                                          const float* bias, int far, float softcap, int window, int chunk,
                                          int num_heads, int num_kv, int head_size, int value_size, int page_pad,
-                                         hipStream_t stream) {
+                                         int splits, float* partial, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_scored_mfma: bad head counts");
+  TNX_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || partial),
+              "attention_scored_mfma: %d blocks a decoded token need a workspace", splits);
   TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention_scored_mfma: bad distance between pages");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
               "attention_scored_mfma: head size %d is not a multiple of 16 in [16, 256]", head_size);
@@ -563,14 +613,12 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
   if (num_single > 0) {
     const int ndb = head_size <= 64 ? 4 : head_size <= 128 ? 8 : 16;
     const size_t parts = (size_t)(SINGLE_WAVES - 1) * 16 * (16 * ndb + 4) * sizeof(float);
-    // query heads a block: 16 (or all), halved while the blocks are fewer than the chip's compute units
-    int width = pack < 16 ? pack : 16;
-    while (width > 1 && (long long)num_single * num_kv * ((pack + width - 1) / width) < 256) width = (width + 1) / 2;
+    const int width = pack < 16 ? pack : 16;      // query heads a block
     const size_t rows = bias ? (size_t)width * (far + 1) * sizeof(float) : 0;
     const size_t most = 160 * 1024;
     const int in_lds = bias && parts + rows <= most;
     const size_t lds = parts + (in_lds ? rows : 0);
-    dim3 grid((unsigned)num_single, (unsigned)num_kv, (unsigned)((pack + width - 1) / width));
+    dim3 grid((unsigned)num_single * splits, (unsigned)num_kv, (unsigned)((pack + width - 1) / width));
 #define LAUNCH_SINGLE(NDB)                                                                                       \
   {                                                                                                              \
     static bool configured = false;                                                                              \
@@ -581,7 +629,7 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
       configured = true;                                                                                         \
     }                                                                                                            \
     attention_scored_single_kernel<NDB><<<grid, 64 * SINGLE_WAVES, lds, stream>>>(a, run_start, cached_lens,     \
-                                                                                   single_runs, width, in_lds, vector_store); \
+                                                                                   single_runs, width, splits, partial, in_lds, vector_store); \
   }
     if (ndb == 4) {
       LAUNCH_SINGLE(4)
@@ -592,6 +640,11 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
     }
 #undef LAUNCH_SINGLE
     TNX_CHECK_LAUNCH("attention_scored_single");
+    if (splits > 1) {
+      attention_scored_join_kernel<<<dim3((unsigned)num_single, (unsigned)num_heads), 64, 0, stream>>>(a, run_start, single_runs,
+                                                                                                       splits, partial);
+      TNX_CHECK_LAUNCH("attention_scored_join");
+    }
   }
   return 0;
 }

@@ -160,7 +160,7 @@ _SIGNATURES = {
         "tnx_attention_scored_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_ll,
                                       _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
         "tnx_attention_scored": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_ll, _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -1537,12 +1537,13 @@ class HipOps:
                            int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size, value_size, sets, pad,
                            _stream(), work=work)
             if not staged or single.numel():
+                splits, partial = self._scored_splits(ctx, single.numel(), num_heads, num_kv_heads, head_size, window, chunk)
                 self._call("scored", "tnx_attention_scored_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.run_start),
                            _ptr(ctx.cached_lens), _ptr(view.block_table), view.width, view.page_size, num_pages, _ptr(tiles),
                            _ptr(ctx.plan["tile_start"]), 0 if staged else tiles.numel(), QUERY_TILE, _ptr(single),
                            single.numel(), _ptr(out), out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far,
                            float(softcap or 0.0), int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size,
-                           value_size, pad, _stream(), work=None if staged else work)
+                           value_size, pad, splits, _ptr(partial), _stream(), work=None if staged else work)
             return out
         self._call("scored", "tnx_attention_scored", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
@@ -1550,6 +1551,24 @@ class HipOps:
                    float(softcap or 0.0), int(window or 0), int(chunk or 0), t, num_heads, num_kv_heads, head_size,
                    value_size, pad, _stream(), work=work)
         return out
+
+    scored_decode_splits = None       # tests set it: the blocks that share a decoded token's keys
+
+    def _scored_splits(self, ctx, singles, num_heads, num_kv_heads, head_size, window, chunk):
+        """(splits, workspace): how many blocks share the keys of a decoded token's (request, key/value head). A
+        token's time is the latency of a wave's chain of loads (measured: a wave lives some 9 us whether it takes
+        one tile or two, and a compute unit holds one or two such blocks), so the tiles the longest request can see
+        are spread until a wave has one (eight waves a block), as long as every block finds a compute unit free. The result
+        does not depend on the number beyond rounding: a recorded step keeps the one it was recorded with."""
+        if not singles:
+            return 1, None
+        longest = ctx.length_bound if ctx.length_bound is not None else ctx.plan_host.get("longest_decode", 0)
+        seen = min(longest, (window or longest) + 63, (chunk or longest) + 63)
+        tiles = seen // 64 + 1
+        splits = self.scored_decode_splits or max(1, min(8, -(-tiles // 8), self.compute_units // max(1, singles * num_kv_heads * -(-(num_heads // num_kv_heads) // 16))))
+        if splits == 1:
+            return 1, None
+        return splits, torch.empty(singles * num_heads * splits * (head_size + 4), dtype=torch.float32, device=self.device)
 
     @staticmethod
     def _scored_work(ctx, num_heads, num_kv_heads, head_size, window, chunk, item):
