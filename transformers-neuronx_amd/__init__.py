@@ -1,4 +1,4 @@
-"""An inference engine for decoder-only language models (OPT, Ratesun, Sunatar, Tadolix) on one AMD MI355X."""
+"""An inference engine for decoder-only language models (OPT, Ratesun, Sunatar, Tadolix, Zotunex) on one AMD MI355X."""
 __version__ = "0.1.0"
 
 from .config import ContinuousBatchingConfig, EngineConfig, GenerationConfig, NeuronConfig  # noqa: F401
@@ -19,6 +19,9 @@ def __getattr__(name):
     if name == "TadolixForSampling":
         from .tadolix import model
         return model.TadolixForSampling
+    if name == "ZotunexForSampling":
+        from .zotunex import model
+        return model.ZotunexForSampling
     if name == "NeuronAutoModelForCausalLM":
         from .modeling_auto import NeuronAutoModelForCausalLM
         return NeuronAutoModelForCausalLM

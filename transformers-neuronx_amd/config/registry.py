@@ -41,7 +41,8 @@ _ARCHITECTURES: Dict[str, Architecture] = {}
 # packages from outside through the environment: TNX_ARCHITECTURE_PACKAGES holds module names, separated
 # by commas, that are importable from where it runs.
 ARCHITECTURE_PACKAGES: List[str] = ["transformers_neuronx_amd.opt", "transformers_neuronx_amd.ratesun",
-                                    "transformers_neuronx_amd.sunatar", "transformers_neuronx_amd.tadolix"]
+                                    "transformers_neuronx_amd.sunatar", "transformers_neuronx_amd.tadolix",
+                                    "transformers_neuronx_amd.zotunex"]
 PACKAGES_VARIABLE = "TNX_ARCHITECTURE_PACKAGES"
 
 

@@ -552,6 +552,7 @@ struct ScoreMods {
   long long gate_ld, out_ld;
   float out_scale;
   int value_size, vector_store;
+  int gate_head;            // the gate's numbers a head: value_size (one an element) or 1 (one for the whole head)
 };
 
 __device__ __forceinline__ int first_visible_key(int pos, int window, int chunk) {
@@ -947,7 +948,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
     if (SCORED) {
       const float inv = sm.out_scale / l[qb];
       bf16_t* orow = out + (size_t)(t0 + qi) * sm.out_ld + h * head_size;
-      const float* gate = sm.gate ? sm.gate + (size_t)(t0 + qi) * sm.gate_ld + (size_t)h * sm.value_size : nullptr;
+      const float* gate = sm.gate ? sm.gate + (size_t)(t0 + qi) * sm.gate_ld + (size_t)h * sm.gate_head : nullptr;
 #pragma unroll
       for (int db = 0; db < NDB; ++db) {
         if (db >= ndb) continue;
@@ -956,7 +957,8 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           float x = o[db][qb][i] * inv;
-          if (gate && d0 + i < sm.value_size) x *= __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gate[d0 + i] * LOG2E));
+          if (gate && d0 + i < sm.value_size)
+            x *= __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gate[sm.gate_head == 1 ? 0 : d0 + i] * LOG2E));
           v4[i] = (bf16_t)x;
         }
         if (sm.vector_store) {
@@ -1622,7 +1624,8 @@ extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, 
                                             int query_tile, void* out, long long out_ld, float out_scale,
                                             const float* gate, long long gate_ld, const float* bias, int far,
                                             float softcap, int window, int chunk, int num_heads, int num_kv,
-                                            int head_size, int value_size, int sets, int page_pad, hipStream_t stream) {
+                                            int head_size, int value_size, int sets, int page_pad, int gate_head,
+                                            hipStream_t stream) {
   TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention_prefill_scored: bad distance between pages");
   TNX_REQUIRE(query_tile == PREFILL_Q_TILE, "attention_prefill_scored: tiles of %d queries, the kernels take %d",
               query_tile, PREFILL_Q_TILE);
@@ -1634,7 +1637,8 @@ extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, 
   TNX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
               "attention_prefill_scored: page size %d is not a power of two from 16 on", page_size);
   TNX_REQUIRE(out_ld >= (long long)num_heads * head_size, "attention_prefill_scored: result rows of %lld elements", out_ld);
-  TNX_REQUIRE(!gate || gate_ld >= (long long)num_heads * value_size, "attention_prefill_scored: gate rows of %lld elements", gate_ld);
+  TNX_REQUIRE(!gate || ((gate_head == 1 || gate_head == value_size) && gate_ld >= (long long)num_heads * gate_head),
+              "attention_prefill_scored: gate rows of %lld elements, %d a head", gate_ld, gate_head);
   TNX_REQUIRE(!bias || far >= 0, "attention_prefill_scored: a bias table needs its last distance");
   TNX_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attention_prefill_scored: bad window, chunk or cap");
   if (num_tiles <= 0) return 0;
@@ -1643,7 +1647,7 @@ extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, 
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   ScoreMods sm{softcap, bias, far, 0, chunk, gate, gate_ld, out_ld, out_scale, value_size,
-               out_ld % 4 == 0 && ((uintptr_t)out & 7) == 0};
+               out_ld % 4 == 0 && ((uintptr_t)out & 7) == 0, gate_head};
   int rc = -1;
 #define SCORED_ARGS                                                                                              \
   grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, \

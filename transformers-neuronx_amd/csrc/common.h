@@ -19,6 +19,7 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 #define TNX_ACT_RELU 1
 #define TNX_ACT_GELU 2      // 0.5 x (1 + erf(x / sqrt 2))
 #define TNX_ACT_GELU_NEW 3  // 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+#define TNX_ACT_RELU2 5     // max(x, 0)^2  (4 is a gated expert's silu)
 
 #define TNX_WAVE 64
 
@@ -161,9 +162,30 @@ __device__ __forceinline__ float apply_act(float x, int act) {
       const float inner = 0.79788456080286535588f * (x + 0.044715f * x * x * x);
       return 0.5f * x * (1.f + tanhf(inner));
     }
+    case TNX_ACT_RELU2: {
+      const float r = fmaxf(x, 0.f);
+      return r * r;
+    }
     default:
       return x;
   }
+}
+
+// What a softmax's running maximum `m` and sum `l` (of exp(score - m) over the visible keys) make of the weighted
+// sum that was gathered with them: the factor 1 / l. With a sink (`sink` non-null: the head's number) the
+// denominator holds exp(sink) once more, with no key and no value behind it; with a gate (`gate` non-null: the
+// (token, head)'s number) the result is multiplied by sigmoid(gate). Full-precision exponentials: once a row.
+__device__ __forceinline__ float softmax_finish(float m, float l, const float* sink, const float* gate) {
+  float f;
+  if (sink != nullptr) {
+    const float s = *sink, top = fmaxf(m, s);
+    const float a = m == -INFINITY ? 0.f : expf(m - top);
+    f = a / (l * a + expf(s - top));
+  } else {
+    f = l > 0.f ? 1.f / l : 0.f;
+  }
+  if (gate != nullptr) f *= 1.f / (1.f + expf(-*gate));
+  return f;
 }
 
 // the compute units of the current device (asked once a device)

@@ -9,6 +9,7 @@
 TNX_DEFINE_ERROR_API
 
 #define TNX_ACT_SILU 4
+#define TNX_ACT_CLAMPED_SWIGLU 6
 
 namespace {
 
@@ -17,13 +18,26 @@ __device__ __forceinline__ float gate_act(float x, int act) {
   return apply_act(x, act);
 }
 
+// What a gated expert makes of the two halves of its first product: act(g) * u; the clamped form, with
+// g' = min(g, limit) and u' = clamp(u, -limit, limit): g' sigmoid(1.702 g') (u' + 1).
+__device__ __forceinline__ float gated(float g, float u, int act, float limit) {
+  if (act == TNX_ACT_CLAMPED_SWIGLU) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+  }
+  return gate_act(g, act) * u;
+}
+
 // ---------------------------------------------------------------- the router's choice
 // A wave a token: `top` rounds of the largest logit (the lower number where two are equal), whose score sigmoid(z)
 // or softmax(z) is the weight. The ranking is by the logits, which both scores grow with: two large logits that
-// float32 still tells apart can have scores that it does not.
+// float32 still tells apart can have scores that it does not. With `correction` (a number an expert) the ranking is
+// by score + correction, and the weight is the score without it; `scale` multiplies every weight.
 __global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z, int tokens, int experts, int top,
                                                     int softmax, int renormalize, int* __restrict__ chosen,
-                                                    float* __restrict__ weights) {
+                                                    float* __restrict__ weights, const float* __restrict__ correction,
+                                                    float scale) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
   if (t >= tokens) return;
   const float* row = z + (size_t)t * experts;
@@ -36,22 +50,23 @@ __global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z,
     total = wave_sum(s);
   }
   auto score = [&](float z) { return softmax ? expf(z - peak) / total : 1.f / (1.f + expf(-z)); };
+  auto rank = [&](int e) { return correction ? score(row[e]) + correction[e] : row[e]; };
   float sum = 0.f;
   unsigned long long taken = 0;        // bit i: expert lane + 64 i is chosen already (a lane's own experts)
   for (int c = 0; c < top; ++c) {
     float best = -INFINITY;
     int at = experts;
     for (int e = lane, i = 0; e < experts; e += 64, ++i) {
-      const float z = row[e];
+      const float z = rank(e);
       if (!((taken >> i) & 1) && (z > best || at == experts)) best = z, at = e;   // ascending e: the lower number stays where two are equal
     }
     const float high = wave_max(best);
     const int first = -(int)wave_max((float)-((best == high && at < experts) ? at : experts));
     if ((first & 63) == lane) taken |= 1ull << (first >> 6);
-    const float s = score(high);
+    const float s = correction ? score(row[first]) : score(high);
     if (lane == 0) {
       chosen[(size_t)t * top + c] = first;
-      weights[(size_t)t * top + c] = renormalize ? 0.f : s;
+      weights[(size_t)t * top + c] = renormalize ? 0.f : s * scale;
     }
     sum += s;
   }
@@ -62,13 +77,13 @@ __global__ void __launch_bounds__(256) route_kernel(const float* __restrict__ z,
       float best = -INFINITY;
       int at = experts;
       for (int e = lane, i = 0; e < experts; e += 64, ++i) {
-        const float z = row[e];
+        const float z = rank(e);
         if (!((taken >> i) & 1) && (z > best || at == experts)) best = z, at = e;
       }
       const float high = wave_max(best);
       const int first = -(int)wave_max((float)-((best == high && at < experts) ? at : experts));
       if ((first & 63) == lane) taken |= 1ull << (first >> 6);
-      if (lane == 0) weights[(size_t)t * top + c] = score(high) / sum;
+      if (lane == 0) weights[(size_t)t * top + c] = (correction ? score(row[first]) : score(high)) / sum * scale;
     }
   }
 }
@@ -126,6 +141,7 @@ struct ProductArgs {
   const float* residual;    // [T, N] or null (not GATED, one choice a token)
   void* out;
   int experts, top, n, k, act, weight_on_input, pairs;
+  float limit;              // of the clamped activation
 };
 
 template <typename T, bool GATED>
@@ -193,7 +209,7 @@ __global__ void __launch_bounds__(256) expert_product_kernel(ProductArgs p) {
     if (GATED) {
       float g = acc[0][r], u = acc[GATED ? 1 : 0][r];
       if (p.weight_on_input) g *= w, u *= w;
-      ((T*)p.out)[(size_t)pair * p.n + col] = from_f32<T>(gate_act(g, p.act) * u);
+      ((T*)p.out)[(size_t)pair * p.n + col] = from_f32<T>(gated(g, u, p.act, p.limit));
     } else {
       float y = acc[0][r];
       if (!p.weight_on_input) y *= w;
@@ -280,7 +296,7 @@ __global__ void __launch_bounds__(256) expert_product_mfma_kernel(ProductArgs p)
     if (GATED) {
       float gt = acc[i], up = acc_up[i];
       if (p.weight_on_input) gt *= w, up *= w;
-      ((bf16_t*)p.out)[(size_t)pair * p.n + col] = (bf16_t)(gate_act(gt, p.act) * up);
+      ((bf16_t*)p.out)[(size_t)pair * p.n + col] = (bf16_t)gated(gt, up, p.act, p.limit);
     } else {
       float y = acc[i];
       if (!p.weight_on_input) y *= w;
@@ -312,13 +328,13 @@ __global__ void combine_kernel(const float* __restrict__ y, const float* __restr
 // (`row_weights`: a factor a row on both g and u, the weight on an expert's input)
 template <typename T>
 __global__ void gated_activation_kernel(const float* __restrict__ gu, T* __restrict__ out, int f, int act, size_t total,
-                                        const float* __restrict__ row_weights) {
+                                        const float* __restrict__ row_weights, float limit) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t stride = (size_t)gridDim.x * blockDim.x;
   for (; i < total; i += stride) {
     const size_t t = i / f, j = i - t * f;
     const float w = row_weights ? row_weights[t] : 1.f;
-    out[i] = from_f32<T>(gate_act(w * gu[t * 2 * f + j], act) * (w * gu[t * 2 * f + f + j]));
+    out[i] = from_f32<T>(gated(w * gu[t * 2 * f + j], w * gu[t * 2 * f + f + j], act, limit));
   }
 }
 
@@ -330,10 +346,11 @@ int blocks_for(size_t total) {
 }  // namespace
 
 extern "C" int tnx_route(const float* z, int tokens, int experts, int top, int softmax, int renormalize, int* chosen,
-                         float* weights, hipStream_t stream) {
+                         float* weights, const float* correction, float scale, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && top <= experts, "route: %d of %d experts", top, experts);
   if (tokens == 0) return 0;
-  route_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(z, tokens, experts, top, softmax, renormalize, chosen, weights);
+  route_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(z, tokens, experts, top, softmax, renormalize, chosen, weights,
+                                                     correction, scale);
   TNX_CHECK_LAUNCH("route");
   return 0;
 }
@@ -341,7 +358,8 @@ extern "C" int tnx_route(const float* z, int tokens, int experts, int top, int s
 extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float* weights, const void* w_gate_up,
                                   const void* w_down, int* first, int* order, void* inner, float* pair_rows,
                                   const float* residual, float* out, int dtype, int tokens, int experts, int top,
-                                  int width, int f, int act, int weight_on_input, int plain, hipStream_t stream) {
+                                  int width, int f, int act, int weight_on_input, int plain, float limit,
+                                  hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && experts > 0 && top > 0 && width > 0 && f > 0, "expert_mixture: bad sizes");
   TNX_REQUIRE(experts <= 4096, "expert_mixture: up to 4096 experts, got %d", experts);
   TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "expert_mixture: dtype %d", dtype);
@@ -352,9 +370,10 @@ extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float*
                                                                top, nullptr, nullptr);
   TNX_CHECK_LAUNCH("expert order");
   const int tiles = pairs / 16 + experts;       // the most tiles of 16 pairs: every expert may end in a part of one
-  ProductArgs up{h, w_gate_up, first, order, weights, nullptr, inner, experts, top, f, width, act, weight_on_input, pairs};
+  ProductArgs up{h, w_gate_up, first, order, weights, nullptr, inner, experts, top, f, width, act, weight_on_input, pairs,
+                 limit};
   ProductArgs down{inner, w_down, first, order, weights, residual, top == 1 ? out : pair_rows, experts, top, width, f,
-                   act, weight_on_input, pairs};
+                   act, weight_on_input, pairs, limit};
   const dim3 grid_up((f + 63) / 64, tiles), grid_down((width + 63) / 64, tiles);
   if (dtype == TNX_F32) {
     expert_product_kernel<float, true><<<grid_up, 256, 0, stream>>>(up);
@@ -377,16 +396,16 @@ extern "C" int tnx_expert_mixture(const void* h, const int* chosen, const float*
 }
 
 extern "C" int tnx_gated_activation(const float* gate_up, void* out, int dtype, int tokens, int f, int act,
-                                    const float* row_weights, hipStream_t stream) {
+                                    const float* row_weights, float limit, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && f > 0, "gated_activation: bad sizes");
   TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "gated_activation: dtype %d", dtype);
   if (tokens == 0) return 0;
   const size_t total = (size_t)tokens * f;
   if (dtype == TNX_F32)
-    gated_activation_kernel<float><<<blocks_for(total), 256, 0, stream>>>(gate_up, (float*)out, f, act, total, row_weights);
+    gated_activation_kernel<float><<<blocks_for(total), 256, 0, stream>>>(gate_up, (float*)out, f, act, total, row_weights, limit);
   else
     gated_activation_kernel<bf16_t><<<blocks_for(total), 256, 0, stream>>>(gate_up, (bf16_t*)out, f, act, total,
-                                                                            row_weights);
+                                                                            row_weights, limit);
   TNX_CHECK_LAUNCH("gated_activation");
   return 0;
 }

@@ -17,11 +17,11 @@ __device__ __forceinline__ void turn_pair(float u, float v, int position, float 
 
 // ------------------------------------------------------------------------------------------------ latents
 
-// One block a token. `down[t]` = [Q | R | r] float32: the first Q, scaled to unit root mean square and
+// One block a token. `down[t]` = [Q | R | r] float32 (rows `ld` elements apart, which may hold more): the first Q, scaled to unit root mean square and
 // weighted, go to `c_q`; the next R likewise to the token's place in the latent pages; the last r, pairs
 // (2i, 2i + 1) turned for i < pairs, to its place in the rotated pages. R = 0: a mixer without a latent of its own.
 __global__ void __launch_bounds__(256)
-latent_norms_kernel(const float* __restrict__ down, int q_rank, int kv_rank, int rot, const float* __restrict__ q_w,
+latent_norms_kernel(const float* __restrict__ down, int ld, int q_rank, int kv_rank, int rot, const float* __restrict__ q_w,
                     const float* __restrict__ kv_w, float eps, const float* __restrict__ freqs, int pairs,
                     const int* __restrict__ positions, const int* __restrict__ token_page,
                     const int* __restrict__ token_offset, void* __restrict__ c_q, int dtype,
@@ -30,11 +30,13 @@ latent_norms_kernel(const float* __restrict__ down, int q_rank, int kv_rank, int
                     int page_size) {
   __shared__ float scratch[4];
   const int t = blockIdx.x;
-  const float* row = down + (size_t)t * (q_rank + kv_rank + rot);
+  const float* row = down + (size_t)t * ld;
   float s = 0.f;
-  for (int i = threadIdx.x; i < q_rank; i += 256) s += row[i] * row[i];
-  const float rq = 1.f / sqrtf(block_sum<4>(s, scratch) / (float)q_rank + eps);
-  for (int i = threadIdx.x; i < q_rank; i += 256) store_any(c_q, dtype, (size_t)t * q_rank + i, row[i] * rq * q_w[i]);
+  if (q_rank > 0) {      // (0: a mixer without a query latent)
+    for (int i = threadIdx.x; i < q_rank; i += 256) s += row[i] * row[i];
+    const float rq = 1.f / sqrtf(block_sum<4>(s, scratch) / (float)q_rank + eps);
+    for (int i = threadIdx.x; i < q_rank; i += 256) store_any(c_q, dtype, (size_t)t * q_rank + i, row[i] * rq * q_w[i]);
+  }
   if (kv_rank == 0) return;
   const int page = token_page[t];
   if (page < 0 || page >= num_pages) return;  // the host checks that every token has a page
@@ -60,19 +62,21 @@ latent_norms_kernel(const float* __restrict__ down, int q_rank, int kv_rank, int
   }
 }
 
-extern "C" int tnx_latent_norms(const float* down, int q_rank, int kv_rank, int rot, const float* q_w,
+extern "C" int tnx_latent_norms(const float* down, int ld, int q_rank, int kv_rank, int rot, const float* q_w,
                                 const float* kv_w, float eps, const float* freqs, int pairs, const int* positions,
                                 const int* token_page, const int* token_offset, void* c_q, int dtype,
                                 void* latent_pages, void* rotated_pages, long long latent_stride,
                                 long long rotated_stride, int num_pages, int page_size, void* across_pages,
                                 long long across_stride, int tokens, hipStream_t stream) {
-  TNX_REQUIRE(tokens >= 0 && q_rank > 0 && kv_rank >= 0 && rot >= 0 && rot % 2 == 0 && (kv_rank == 0 || 2 * pairs <= rot),
+  TNX_REQUIRE(tokens >= 0 && q_rank >= 0 && kv_rank >= 0 && q_rank + kv_rank > 0 && rot >= 0 && rot % 2 == 0 &&
+                  (kv_rank == 0 || 2 * pairs <= rot) && (q_rank == 0 || (q_w && c_q)),
               "latent_norms: bad sizes q=%d kv=%d rot=%d pairs=%d", q_rank, kv_rank, rot, pairs);
+  TNX_REQUIRE(ld >= q_rank + kv_rank + (kv_rank ? rot : 0), "latent_norms: rows of %d elements", ld);
   TNX_REQUIRE(kv_rank == 0 || (latent_pages && rotated_pages && kv_w && latent_stride >= (long long)page_size * kv_rank &&
                                rotated_stride >= (long long)page_size * rot),
               "latent_norms: pages too small for their tokens");
   if (tokens == 0) return 0;
-  latent_norms_kernel<<<tokens, 256, 0, stream>>>(down, q_rank, kv_rank, kv_rank ? rot : 0, q_w, kv_w, eps, freqs, pairs,
+  latent_norms_kernel<<<tokens, 256, 0, stream>>>(down, ld, q_rank, kv_rank, kv_rank ? rot : 0, q_w, kv_w, eps, freqs, pairs,
                                                   positions, token_page, token_offset, c_q, dtype, latent_pages,
                                                   rotated_pages, (size_t)latent_stride, (size_t)rotated_stride,
                                                   num_pages, kv_rank ? across_pages : nullptr, (size_t)across_stride,
@@ -205,6 +209,18 @@ extern "C" int tnx_batched_linear(const void* x, int x_dtype, long long x_row, l
   return 0;
 }
 
+// What ends a (query, head)'s softmax beside the division by its sum (`softmax_finish`): a number a head that
+// joins the denominator as exp(sink), and a gate a (token, head) whose sigmoid multiplies the result; either may
+// be absent.
+struct LatentFinish {
+  const float* sink;     // [H] or null
+  const float* gate;     // [T, gate_ld], a number a head, or null
+  long long gate_ld;
+};
+__device__ __forceinline__ float latent_finish(const LatentFinish& f, float m, float l, size_t token, int head) {
+  return softmax_finish(m, l, f.sink ? f.sink + head : nullptr, f.gate ? f.gate + token * f.gate_ld + head : nullptr);
+}
+
 // ------------------------------------------------------------------------------------------------ attention, any sizes
 
 // One block of 256 threads a (token, head). The query's two parts lie in LDS as float32 (q_r turned by the
@@ -219,7 +235,7 @@ latent_attention_any_kernel(const T* __restrict__ q, const T* __restrict__ q_lat
                             const int* __restrict__ block_table, int table_width, int page_size, int num_pages,
                             const T* __restrict__ latent_pages, const T* __restrict__ rotated_pages,
                             size_t latent_stride, size_t rotated_stride, const float* __restrict__ freqs, int pairs,
-                            float scale, int heads, int head_size, int rot, int kv_rank, int window) {
+                            float scale, int heads, int head_size, int rot, int kv_rank, int window, LatentFinish fin) {
   extern __shared__ float lds[];
   float* ql = lds;                 // [kv_rank]
   float* qr = ql + kv_rank;        // [rot]
@@ -290,7 +306,7 @@ latent_attention_any_kernel(const T* __restrict__ q, const T* __restrict__ q_lat
     }
     __syncthreads();
   }
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float inv = latent_finish(fin, m, l, t, h);
 #pragma unroll
   for (int i = 0; i < LA_OWN; ++i) {
     const int d = threadIdx.x + i * 256;
@@ -303,24 +319,27 @@ extern "C" int tnx_latent_attention_any(const void* q, int dtype, const void* q_
                                         int page_size, int num_pages, const void* latent_pages,
                                         const void* rotated_pages, long long latent_stride, long long rotated_stride,
                                         const float* freqs, int pairs, float scale, int heads, int head_size, int rot,
-                                        int kv_rank, int window, int tokens, hipStream_t stream) {
+                                        int kv_rank, int window, int tokens, const float* sink, const float* gate,
+                                        long long gate_ld, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && heads > 0 && heads <= 65535 && kv_rank > 0 && rot >= 0 && rot % 2 == 0 && 2 * pairs <= rot,
               "latent_attention: bad sizes heads=%d kv_rank=%d rot=%d", heads, kv_rank, rot);
   TNX_REQUIRE(kv_rank <= 256 * LA_OWN, "latent_attention: a latent of %d elements is more than %d", kv_rank, 256 * LA_OWN);
   TNX_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0 && window >= 0, "latent_attention: bad page sizes");
   if (tokens == 0) return 0;
+  TNX_REQUIRE(!gate || gate_ld >= heads, "latent_attention: gate rows of %lld elements", gate_ld);
   const size_t lds = (size_t)(kv_rank + rot + 512) * sizeof(float);
   const dim3 grid(tokens, heads);
+  const LatentFinish fin{sink, gate, gate_ld};
   if (dtype == TNX_F32)
     latent_attention_any_kernel<float><<<grid, 256, lds, stream>>>(
         (const float*)q, (const float*)q_lat, (float*)out, positions, token_request, block_table, table_width, page_size,
         num_pages, (const float*)latent_pages, (const float*)rotated_pages, (size_t)latent_stride, (size_t)rotated_stride,
-        freqs, pairs, scale, heads, head_size, rot, kv_rank, window);
+        freqs, pairs, scale, heads, head_size, rot, kv_rank, window, fin);
   else
     latent_attention_any_kernel<bf16_t><<<grid, 256, lds, stream>>>(
         (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, positions, token_request, block_table, table_width,
         page_size, num_pages, (const bf16_t*)latent_pages, (const bf16_t*)rotated_pages, (size_t)latent_stride,
-        (size_t)rotated_stride, freqs, pairs, scale, heads, head_size, rot, kv_rank, window);
+        (size_t)rotated_stride, freqs, pairs, scale, heads, head_size, rot, kv_rank, window, fin);
   TNX_CHECK_LAUNCH("latent_attention_any");
   return 0;
 }
@@ -482,7 +501,7 @@ latent_attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
                                const int* __restrict__ table, int table_width, const int* __restrict__ tile_run,
                                const int* __restrict__ tile_q0, int tile_tokens, LatentPages pg,
                                const float* __restrict__ freqs, int pairs, float scale, int heads, int head_size,
-                               int window) {
+                               int window, LatentFinish fin) {
   constexpr int NKS = (16 * NDB + LM_ROT) / 32;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 15, g = lane >> 4;
@@ -543,7 +562,7 @@ latent_attention_prompt_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   for (int qb = 0; qb < QB; ++qb) {
     const int qi = qw0 + 16 * qb + r;
     if (qi >= qlen) continue;
-    const float inv = l[qb] > 0.f ? 1.f / l[qb] : 0.f;
+    const float inv = latent_finish(fin, m[qb], l[qb], t0 + qi, h);
     bf16_t* orow = out + ((size_t)(t0 + qi) * heads + h) * R;
 #pragma unroll
     for (int db = 0; db < NDB; ++db) {
@@ -569,7 +588,8 @@ latent_attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
                                const int* __restrict__ run_start, const int* __restrict__ cached_lens,
                                const int* __restrict__ table, int table_width, const int* __restrict__ decode_runs,
                                LatentPages pg, const float* __restrict__ freqs, int pairs, float scale, int heads,
-                               int head_size, int window, float* __restrict__ part, int splits, int tiles_per_split) {
+                               int head_size, int window, float* __restrict__ part, int splits, int tiles_per_split,
+                               LatentFinish fin) {
   constexpr int NKS = (16 * NDB + LM_ROT) / 32;
   constexpr int OWN = (NDB + 3) / 4;           // blocks of 16 latent elements a wave owns: wave, wave + 4, ...
   __shared__ float tile_max[4][16], tile_sum[4][16];
@@ -681,7 +701,7 @@ latent_attention_decode_kernel(const bf16_t* __restrict__ q, const bf16_t* __res
   }
   if (h >= heads) return;
   if (splits == 1) {
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    const float inv = latent_finish(fin, m, l, t, h);
     bf16_t* orow = out + ((size_t)t * heads + h) * R;
 #pragma unroll
     for (int j = 0; j < OWN; ++j) {
@@ -721,7 +741,7 @@ latent_attention_prompt_shared_kernel(const bf16_t* __restrict__ q, const bf16_t
                                       int table_width, const int* __restrict__ tile_run,
                                       const int* __restrict__ tile_q0, int tile_tokens, LatentPages pg,
                                       const float* __restrict__ freqs, int pairs, float scale, int heads,
-                                      int head_size, int window) {
+                                      int head_size, int window, LatentFinish fin) {
   constexpr int NKS = (16 * NDB + LM_ROT) / 32;
   constexpr int OWN = (NDB + 3) / 4;
   __shared__ float tile_max[4][HB][16], tile_sum[4][HB][16];
@@ -865,7 +885,7 @@ latent_attention_prompt_shared_kernel(const bf16_t* __restrict__ q, const bf16_t
   for (int hb = 0; hb < HB; ++hb) {
     const int h = HB * hg + hb;
     if (h >= heads) continue;
-    const float inv = l[hb] > 0.f ? 1.f / l[hb] : 0.f;
+    const float inv = latent_finish(fin, m[hb], l[hb], t0 + qi, h);
     bf16_t* orow = out + ((size_t)(t0 + qi) * heads + h) * R;
 #pragma unroll
     for (int j = 0; j < OWN; ++j) {
@@ -882,7 +902,7 @@ latent_attention_prompt_shared_kernel(const bf16_t* __restrict__ q, const bf16_t
 // joins the partial results of the splits of one (decode run, head): one block each
 __global__ void __launch_bounds__(256)
 latent_attention_join_kernel(const float* __restrict__ part, bf16_t* __restrict__ out, const int* __restrict__ run_start,
-                             const int* __restrict__ decode_runs, int heads, int kv_rank, int splits) {
+                             const int* __restrict__ decode_runs, int heads, int kv_rank, int splits, LatentFinish fin) {
   const int h = blockIdx.y;
   const int t = run_start[decode_runs[blockIdx.x]];
   const float* mine = part + ((size_t)blockIdx.x * heads + h) * splits * (kv_rank + 2);
@@ -892,7 +912,7 @@ latent_attention_join_kernel(const float* __restrict__ part, bf16_t* __restrict_
   float l = 0.f;
   for (int s = 0; s < splits; ++s)
     l += mine[(size_t)s * (kv_rank + 2) + kv_rank + 1] * __expf(mine[(size_t)s * (kv_rank + 2) + kv_rank] - m_safe);
-  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const float inv = latent_finish(fin, m, l, t, h);
   for (int d = threadIdx.x; d < kv_rank; d += 256) {
     float acc = 0.f;
     for (int s = 0; s < splits; ++s) {
@@ -916,7 +936,7 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
                                          long long rotated_stride, long long across_stride, const float* freqs, int pairs,
                                          float scale, int heads, int head_size, int rot, int kv_rank, int window,
                                          float* part, int splits, int tiles_per_split, int prompt_kind,
-                                         hipStream_t stream) {
+                                         const float* sink, const float* gate, long long gate_ld, hipStream_t stream) {
   TNX_REQUIRE(kv_rank > 0 && kv_rank % 16 == 0 && kv_rank <= 512, "latent_attention_mfma: a latent of %d elements", kv_rank);
   TNX_REQUIRE(rot >= 0 && rot % 8 == 0 && rot <= LM_ROT && 2 * pairs <= rot, "latent_attention_mfma: a rotated part of %d", rot);
   TNX_REQUIRE(page_size > 0 && page_size % 16 == 0 && table_width > 0 && num_pages > 0 && window >= 0 && heads > 0,
@@ -928,20 +948,22 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
               "latent_attention_mfma: %d splits of %d tiles", splits, tiles_per_split);
   TNX_REQUIRE(latent_stride % 8 == 0 && rotated_stride % 8 == 0 && across_stride % 8 == 0,
               "latent_attention_mfma: pages that are not aligned");
+  TNX_REQUIRE(!gate || gate_ld >= heads, "latent_attention_mfma: gate rows of %lld elements", gate_ld);
+  const LatentFinish fin{sink, gate, gate_ld};
   LatentPages pg = {(const bf16_t*)latent_pages, (const bf16_t*)rotated_pages, (const bf16_t*)across_pages,
                     (size_t)latent_stride, (size_t)rotated_stride, (size_t)across_stride, page_size, num_pages, kv_rank, rot};
 #define LM_PROMPT(NDB, QB)                                                                                             \
   latent_attention_prompt_kernel<NDB, QB><<<tiles * (tile_tokens / (64 * QB)) * heads, 256, 0, stream>>>(              \
       (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width, tile_run, \
-      tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window)
+      tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window, fin)
 #define LM_DECODE(NDB)                                                                                          \
   latent_attention_decode_kernel<NDB><<<dim3(decodes, (heads + 15) / 16, splits), 256, 0, stream>>>(            \
       (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width,   \
-      decode_runs, pg, freqs, pairs, scale, heads, head_size, window, part, splits, tiles_per_split)
+      decode_runs, pg, freqs, pairs, scale, heads, head_size, window, part, splits, tiles_per_split, fin)
 #define LM_SHARED(NDB, HB)                                                                                            \
   latent_attention_prompt_shared_kernel<NDB, HB><<<tiles * (tile_tokens / 16) * ((heads + HB - 1) / HB), 256, 0, stream>>>( \
       (const bf16_t*)q, (const bf16_t*)q_lat, (bf16_t*)out, run_start, cached_lens, block_table, table_width, tile_run,   \
-      tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window)
+      tile_q0, tile_tokens, pg, freqs, pairs, scale, heads, head_size, window, fin)
   if (tiles > 0 && prompt_kind == 0) {
     if (kv_rank <= 64) { if (heads >= 4) LM_SHARED(4, 4); else LM_SHARED(4, 1); }
     else if (kv_rank <= 128) { if (heads >= 4) LM_SHARED(8, 4); else LM_SHARED(8, 1); }
@@ -964,7 +986,7 @@ extern "C" int tnx_latent_attention_mfma(const void* q, const void* q_lat, void*
     TNX_CHECK_LAUNCH("latent_attention_decode");
     if (splits > 1) {
       latent_attention_join_kernel<<<dim3(decodes, heads), 256, 0, stream>>>(part, (bf16_t*)out, run_start, decode_runs,
-                                                                            heads, kv_rank, splits);
+                                                                            heads, kv_rank, splits, fin);
       TNX_CHECK_LAUNCH("latent_attention_join");
     }
   }
@@ -1013,7 +1035,8 @@ expanded_attention_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict
                           const int* __restrict__ cached_lens, const int* __restrict__ ctx_start,
                           const int* __restrict__ ctx_base, const int* __restrict__ tile_run,
                           const int* __restrict__ tile_q0, int tile_tokens, size_t rows, const float* __restrict__ freqs,
-                          int pairs, float scale, int heads, int head_size, int rot, int value_size, int window) {
+                          int pairs, float scale, int heads, int head_size, int rot, int value_size, int window,
+                          LatentFinish fin) {
   constexpr int QB = 4;
   constexpr int OWN = (NDV + 3) / 4;
   __shared__ float tile_max[4][QB][16], tile_sum[4][QB][16];
@@ -1146,7 +1169,7 @@ expanded_attention_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict
   for (int qb = 0; qb < QB; ++qb) {
     const int qi = q0 + 16 * qb + r;
     if (qi >= qlen) continue;
-    const float inv = l[qb] > 0.f ? 1.f / l[qb] : 0.f;
+    const float inv = latent_finish(fin, m[qb], l[qb], t0 + qi, h);
     bf16_t* orow = out + ((size_t)(t0 + qi) * heads + h) * value_size;
 #pragma unroll
     for (int j = 0; j < OWN; ++j) {
@@ -1179,22 +1202,24 @@ extern "C" int tnx_expanded_attention(const void* q, const void* k_n, const void
                                       const int* run_start, const int* cached_lens, const int* ctx_start,
                                       const int* ctx_base, const int* tile_run, const int* tile_q0, int tiles,
                                       int tile_tokens, long long rows, const float* freqs, int pairs, float scale,
-                                      int heads, int head_size, int rot, int value_size, int window,
-                                      hipStream_t stream) {
+                                      int heads, int head_size, int rot, int value_size, int window, const float* sink,
+                                      const float* gate, long long gate_ld, hipStream_t stream) {
   TNX_REQUIRE(tiles >= 0 && heads > 0 && head_size > 0 && head_size % 8 == 0 && rot >= 0 && rot % 8 == 0 &&
                   head_size + rot <= 256 && 2 * pairs <= rot,
               "expanded_attention: query/key sizes %d + %d", head_size, rot);
   TNX_REQUIRE(value_size > 0 && value_size % 16 == 0 && value_size <= 256, "expanded_attention: a value of %d elements", value_size);
   TNX_REQUIRE(tile_tokens == 128 && rows % 64 == 0 && window >= 0, "expanded_attention: tiles of %d queries, %lld rows",
               tile_tokens, rows);
+  TNX_REQUIRE(!gate || gate_ld >= heads, "expanded_attention: gate rows of %lld elements", gate_ld);
   if (tiles == 0) return 0;
+  const LatentFinish fin{sink, gate, gate_ld};
   const int grid = tiles * (tile_tokens / 64) * heads;
   const int nks = (head_size + rot + 31) / 32, ndv = value_size / 16;
 #define EA_LAUNCH(NKS, NDV)                                                                                          \
   expanded_attention_kernel<NKS, NDV><<<grid, 256, 0, stream>>>(                                                     \
       (const bf16_t*)q, (const bf16_t*)k_n, (const bf16_t*)k_r, (const bf16_t*)v_t, (bf16_t*)out, run_start,          \
       cached_lens, ctx_start, ctx_base, tile_run, tile_q0, tile_tokens, (size_t)rows, freqs, pairs, scale, heads,     \
-      head_size, rot, value_size, window)
+      head_size, rot, value_size, window, fin)
 #define EA_VALUES(NKS)                        \
   if (ndv <= 4) { EA_LAUNCH(NKS, 4); }        \
   else if (ndv <= 8) { EA_LAUNCH(NKS, 8); }   \

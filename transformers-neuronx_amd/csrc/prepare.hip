@@ -31,6 +31,8 @@ struct PrepareArgs {
   int num_pages, page_size;
   int heads, groups, n, v, d;
   int per_head;             // every head is normed by itself (the weights, if any, still one a projection element)
+  int values_at;            // the column of a row where the values begin (behind the keys, or the keys' own)
+  const float* head_scale;  // [H] or null: a query head's elements times its number, beside `scale`
 };
 
 // Element `e` of head `head` of a normed projection, turned by the token's position. `x` points at the
@@ -70,7 +72,7 @@ __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
   const int page = a.token_page[t], off = a.token_offset[t];
   if (part > 0 && (page < 0 || page >= a.num_pages)) return;       // the host checks that every token has a page
   if (part == 2) {
-    const float* xv = row + nq + nk;
+    const float* xv = row + a.values_at;
     T* vp = (T*)a.v_pages + (size_t)page * a.page_stride;
     const float lam = a.first != nullptr ? a.mix_weight[0] : 0.f;
     const float* first = a.first != nullptr ? a.first + (size_t)t * a.first_ld : nullptr;
@@ -106,7 +108,7 @@ __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
       for (int e = lane; e < a.d; e += 64) {
         const float val = e < a.n ? turned(x, w, r, head, e, a, cosines, sines) : 0.f;
         if (part == 0)
-          q_out[head * a.d + e] = from_f32<T>(val * a.scale);
+          q_out[head * a.d + e] = from_f32<T>(val * (a.head_scale ? a.scale * a.head_scale[head] : a.scale));
         else
           kp[((size_t)head * a.page_size + off) * a.d + e] = from_f32<T>(val);
       }
@@ -125,7 +127,9 @@ __global__ void __launch_bounds__(256) qkv_prepare_kernel(PrepareArgs a) {
     T* q_out = (T*)a.q_out + (size_t)t * a.heads * a.d;
     for (int i = threadIdx.x; i < heads * a.d; i += 256) {
       const int head = i / a.d, e = i - head * a.d;
-      q_out[i] = from_f32<T>(e < a.n ? turned(x, w, norm, head, e, a, cosines, sines) * a.scale : 0.f);
+      q_out[i] = from_f32<T>(e < a.n ? turned(x, w, norm, head, e, a, cosines, sines) *
+                                           (a.head_scale ? a.scale * a.head_scale[head] : a.scale)
+                                     : 0.f);
     }
   } else {
     T* kp = (T*)a.k_pages + (size_t)page * a.page_stride;
@@ -143,11 +147,12 @@ extern "C" int tnx_qkv_prepare(const float* proj, int ld, const float* q_weight,
                                const float* mix_weight, const float* first, long long first_ld, const int* token_page,
                                const int* token_offset, void* q_out, void* k_pages, void* v_pages, long long page_stride,
                                int num_pages, int page_size, int dtype, int tokens, int heads, int groups, int n, int v,
-                               int d, int per_head, hipStream_t stream) {
+                               int d, int per_head, int values_at, const float* head_scale, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && heads > 0 && groups > 0 && n > 0 && v > 0, "qkv_prepare: bad sizes");
   TNX_REQUIRE(d >= n && d >= v, "qkv_prepare: cached heads of %d elements do not hold %d and %d", d, n, v);
-  TNX_REQUIRE(ld >= heads * n + groups * (n + v), "qkv_prepare: rows of %d elements, %d needed", ld,
-              heads * n + groups * (n + v));
+  if (values_at < 0) values_at = heads * n + groups * n;
+  TNX_REQUIRE(ld >= heads * n + groups * n && ld >= values_at + groups * v,
+              "qkv_prepare: rows of %d elements do not hold the keys and the values at column %d", ld, values_at);
   TNX_REQUIRE(freqs == nullptr || (2 * half <= n && half <= 128), "qkv_prepare: %d turned elements in heads of %d", 2 * half, n);
   TNX_REQUIRE((q_weight == nullptr) == (k_weight == nullptr), "qkv_prepare: both norm weights or none");
   TNX_REQUIRE((first == nullptr) || (mix_weight != nullptr && first_ld >= groups * v), "qkv_prepare: blending needs its weight");
@@ -156,7 +161,7 @@ extern "C" int tnx_qkv_prepare(const float* proj, int ld, const float* q_weight,
   if (tokens == 0) return 0;
   PrepareArgs a{proj, ld, q_weight, k_weight, eps, freqs, half, interleaved, positions, scale, mix_weight, first, first_ld,
                 token_page, token_offset, q_out, k_pages, v_pages, page_stride, num_pages, page_size, heads, groups, n, v, d,
-                per_head};
+                per_head, values_at, head_scale};
   if (dtype == TNX_F32)
     qkv_prepare_kernel<float><<<dim3(tokens, 3), 256, 0, stream>>>(a);
   else

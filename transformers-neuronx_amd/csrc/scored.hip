@@ -25,8 +25,9 @@ struct ScoredArgs {
   void* out;                // [T, out_ld]
   long long out_ld;
   float out_scale;
-  const float* gate;        // [T, gate_ld] or null: pre-activations of the gate, H * value_size a token
+  const float* gate;        // [T, gate_ld] or null: pre-activations of the gate, H * gate_head a token
   long long gate_ld;
+  int gate_head;            // the gate's numbers a head: value_size (one an element) or 1 (one for the whole head)
   const float* bias;        // [H, far + 1] or null
   int far;
   float softcap;            // 0: none
@@ -119,13 +120,13 @@ __global__ void __launch_bounds__(256) attention_scored_any_kernel(ScoredArgs a)
   }
   const float inv = a.out_scale / l;
   T* out = (T*)a.out + (size_t)t * a.out_ld + (size_t)h * head_size;
-  const float* gate = a.gate ? a.gate + (size_t)t * a.gate_ld + (size_t)h * a.value_size : nullptr;
+  const float* gate = a.gate ? a.gate + (size_t)t * a.gate_ld + (size_t)h * a.gate_head : nullptr;
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int d = lane + 64 * e;
     if (d >= head_size) continue;
     float v = acc[e] * inv;
-    if (gate && d < a.value_size) v *= 1.f / (1.f + expf(-gate[d]));
+    if (gate && d < a.value_size) v *= 1.f / (1.f + expf(-gate[a.gate_head == 1 ? 0 : d]));
     out[d] = from_f32<T>(v);
   }
 }
@@ -302,12 +303,12 @@ __device__ __forceinline__ void scored_walk(const ScoredArgs& a, const int* __re
 __device__ __forceinline__ void store_four(const ScoredArgs& a, int token, int head, int d0, f32x4 v, float scale,
                                            bool vector_store) {
   bf16_t* orow = (bf16_t*)a.out + (size_t)token * a.out_ld + (size_t)head * a.head_size + d0;
-  const float* gate = a.gate ? a.gate + (size_t)token * a.gate_ld + (size_t)head * a.value_size : nullptr;
+  const float* gate = a.gate ? a.gate + (size_t)token * a.gate_ld + (size_t)head * a.gate_head : nullptr;
   bf16x4 v4;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     float x = v[i] * scale;
-    if (gate && d0 + i < a.value_size) x *= __builtin_amdgcn_rcpf(1.f + __expf(-gate[d0 + i]));
+    if (gate && d0 + i < a.value_size) x *= __builtin_amdgcn_rcpf(1.f + __expf(-gate[a.gate_head == 1 ? 0 : d0 + i]));
     v4[i] = (bf16_t)x;
   }
   if (vector_store) {
@@ -515,7 +516,7 @@ attention_scored_join_kernel(ScoredArgs a, const int* __restrict__ run_start, co
     ll += ms == -INFINITY ? 0.f : mine[s * stride + 1] * __expf(ms - mm);
   }
   bf16_t* orow = (bf16_t*)a.out + (size_t)token * a.out_ld + (size_t)head * a.head_size;
-  const float* gate = a.gate ? a.gate + (size_t)token * a.gate_ld + (size_t)head * a.value_size : nullptr;
+  const float* gate = a.gate ? a.gate + (size_t)token * a.gate_ld + (size_t)head * a.gate_head : nullptr;
   for (int d = threadIdx.x; d < a.head_size; d += 64) {
     float oo = 0.f;
     for (int s = 0; s < splits; ++s) {
@@ -523,7 +524,7 @@ attention_scored_join_kernel(ScoredArgs a, const int* __restrict__ run_start, co
       if (ms != -INFINITY) oo += mine[s * stride + 4 + d] * __expf(ms - mm);
     }
     float x = oo * a.out_scale / ll;
-    if (gate && d < a.value_size) x *= 1.f / (1.f + __expf(-gate[d]));
+    if (gate && d < a.value_size) x *= 1.f / (1.f + __expf(-gate[a.gate_head == 1 ? 0 : d]));
     orow[d] = (bf16_t)x;
   }
 }
@@ -535,7 +536,7 @@ extern "C" int tnx_attention_scored(const void* q, int dtype, const void* k_page
                                     int page_size, int num_pages, void* out, long long out_ld, float out_scale,
                                     const float* gate, long long gate_ld, const float* bias, int far, float softcap,
                                     int window, int chunk, int tokens, int num_heads, int num_kv, int head_size,
-                                    int value_size, int page_pad, hipStream_t stream) {
+                                    int value_size, int page_pad, int gate_head, hipStream_t stream) {
   TNX_REQUIRE(tokens >= 0 && num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_scored: bad head counts");
   TNX_REQUIRE(page_pad >= 0 && page_pad % 8 == 0, "attention_scored: bad distance between pages");
   TNX_REQUIRE(head_size % 16 == 0 && head_size >= 16 && head_size <= 256,
@@ -543,7 +544,8 @@ extern "C" int tnx_attention_scored(const void* q, int dtype, const void* k_page
   TNX_REQUIRE(value_size > 0 && value_size <= head_size, "attention_scored: values of %d in heads of %d", value_size, head_size);
   TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention_scored: page size %d is not a multiple of 16", page_size);
   TNX_REQUIRE(out_ld >= (long long)num_heads * head_size, "attention_scored: result rows of %lld elements", out_ld);
-  TNX_REQUIRE(!gate || gate_ld >= (long long)num_heads * value_size, "attention_scored: gate rows of %lld elements", gate_ld);
+  TNX_REQUIRE(!gate || ((gate_head == 1 || gate_head == value_size) && gate_ld >= (long long)num_heads * gate_head),
+              "attention_scored: gate rows of %lld elements, %d a head", gate_ld, gate_head);
   TNX_REQUIRE(!bias || far >= 0, "attention_scored: a bias table needs its last distance");
   TNX_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attention_scored: bad window, chunk or cap");
   TNX_REQUIRE(dtype == TNX_F32 || dtype == TNX_BF16, "attention_scored: dtype %d", dtype);
@@ -552,7 +554,7 @@ extern "C" int tnx_attention_scored(const void* q, int dtype, const void* k_page
   const long long blocks = (waves + 3) / 4;
   TNX_REQUIRE(blocks < (1ll << 31), "attention_scored: too many (token, head) pairs");
   ScoredArgs a{q, k_pages, v_pages, positions, token_request, table, table_width, page_size, num_pages, out, out_ld,
-               out_scale, gate, gate_ld, bias, far, softcap, window, chunk, tokens, num_heads, num_kv, head_size,
+               out_scale, gate, gate_ld, gate_head, bias, far, softcap, window, chunk, tokens, num_heads, num_kv, head_size,
                value_size, page_pad};
   if (dtype == TNX_F32)
     attention_scored_any_kernel<float><<<(unsigned)blocks, 256, 0, stream>>>(a);
@@ -571,7 +573,7 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
                                          long long out_ld, float out_scale, const float* gate, long long gate_ld,
                                          const float* bias, int far, float softcap, int window, int chunk,
                                          int num_heads, int num_kv, int head_size, int value_size, int page_pad,
-                                         int splits, float* partial, hipStream_t stream) {
+                                         int splits, float* partial, int gate_head, hipStream_t stream) {
   TNX_REQUIRE(num_heads > 0 && num_kv > 0 && num_heads % num_kv == 0, "attention_scored_mfma: bad head counts");
   TNX_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || partial),
               "attention_scored_mfma: %d blocks a decoded token need a workspace", splits);
@@ -581,14 +583,15 @@ extern "C" int tnx_attention_scored_mfma(const void* q, const void* k_pages, con
   TNX_REQUIRE(value_size > 0 && value_size <= head_size, "attention_scored_mfma: values of %d in heads of %d", value_size, head_size);
   TNX_REQUIRE(page_size % 16 == 0 && page_size > 0, "attention_scored_mfma: page size %d is not a multiple of 16", page_size);
   TNX_REQUIRE(out_ld >= (long long)num_heads * head_size, "attention_scored_mfma: result rows of %lld elements", out_ld);
-  TNX_REQUIRE(!gate || gate_ld >= (long long)num_heads * value_size, "attention_scored_mfma: gate rows of %lld elements", gate_ld);
+  TNX_REQUIRE(!gate || ((gate_head == 1 || gate_head == value_size) && gate_ld >= (long long)num_heads * gate_head),
+              "attention_scored_mfma: gate rows of %lld elements, %d a head", gate_ld, gate_head);
   TNX_REQUIRE(!bias || far >= 0, "attention_scored_mfma: a bias table needs its last distance");
   TNX_REQUIRE(window >= 0 && chunk >= 0 && softcap >= 0.f, "attention_scored_mfma: bad window, chunk or cap");
   TNX_REQUIRE(num_tiles <= 0 || query_tile == 128, "attention_scored_mfma: tiles of %d queries, the kernel takes 128", query_tile);
   TNX_REQUIRE((long long)(num_tiles > 0 ? num_tiles : 0) * num_heads < (1ll << 31), "attention_scored_mfma: too many tiles");
   TNX_REQUIRE(num_single < 65536 * 1024 && num_kv < 65536, "attention_scored_mfma: too many runs or heads");
   ScoredArgs a{q, k_pages, v_pages, nullptr, nullptr, table, table_width, page_size, num_pages, out, out_ld,
-               out_scale, gate, gate_ld, bias, far, softcap, window, chunk, 0, num_heads, num_kv, head_size,
+               out_scale, gate, gate_ld, gate_head, bias, far, softcap, window, chunk, 0, num_heads, num_kv, head_size,
                value_size, page_pad};
   const int vector_store = out_ld % 4 == 0 && ((uintptr_t)out & 7) == 0;
   const int pack = num_heads / num_kv;

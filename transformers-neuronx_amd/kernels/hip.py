@@ -16,8 +16,8 @@ from .attention_plan import QUERY_TILE
 from .. import debug
 
 _F32, _BF16 = 0, 1
-_ACT = {None: 0, "none": 0, "relu": 1, "gelu": 2, "gelu_new": 3}
-_GATE_ACT = {"gelu_new": 3, "silu": 4}     # what a gated expert's kernels take
+_ACT = {None: 0, "none": 0, "relu": 1, "gelu": 2, "gelu_new": 3, "relu2": 5}
+_GATE_ACT = {"gelu_new": 3, "silu": 4, "clamped_swiglu": 6}     # what a gated expert's kernels take
 _LIBS: Dict[str, ctypes.CDLL] = {}
 
 _c_void_p, _c_int, _c_float, _c_ll = ctypes.c_void_p, ctypes.c_int, ctypes.c_float, ctypes.c_longlong
@@ -64,7 +64,7 @@ _SIGNATURES = {
         "tnx_attention_prefill_scored": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                          _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_ll, _c_float,
                                          _c_void_p, _c_ll, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_int, _c_int,
-                                         _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                         _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_attention_prefill": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                   _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_int,
                                   _c_int, _c_int, _c_int, _c_void_p],
@@ -102,29 +102,31 @@ _SIGNATURES = {
         "tnx_weighted_sum": [_c_void_p, _c_void_p, _c_int, _c_ll, _c_void_p, _c_ll, _c_void_p],
     },
     "latent": {
-        "tnx_latent_norms": [_c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int,
+        "tnx_latent_norms": [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int,
                              _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll,
                              _c_int, _c_int, _c_void_p, _c_ll, _c_int, _c_void_p],
         "tnx_latent_attention_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p,
                                       _c_void_p, _c_void_p, _c_ll, _c_ll, _c_ll, _c_void_p, _c_int, _c_float, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
+                                      _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_int, _c_void_p,
+                                      _c_void_p, _c_ll, _c_void_p],
         "tnx_batched_linear": [_c_void_p, _c_int, _c_ll, _c_ll, _c_void_p, _c_int, _c_void_p, _c_int, _c_float, _c_int,
                                _c_int, _c_int, _c_int, _c_void_p],
         "tnx_latent_gather": [_c_void_p, _c_void_p, _c_ll, _c_ll, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_void_p,
                               _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
         "tnx_expanded_attention": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                    _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_ll, _c_void_p, _c_int, _c_float,
-                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_ll, _c_void_p],
         "tnx_latent_attention_any": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int,
                                      _c_int, _c_int, _c_void_p, _c_void_p, _c_ll, _c_ll, _c_void_p, _c_int, _c_float,
-                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_ll,
+                                     _c_void_p],
     },
     "prepare": {
         "tnx_qkv_prepare": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_void_p,
                             _c_float, _c_void_p, _c_void_p, _c_ll, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                             _c_ll, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                            _c_void_p],
+                            _c_int, _c_void_p, _c_void_p],
     },
     "memory": {
         "tnx_matrix_memory": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
@@ -132,11 +134,12 @@ _SIGNATURES = {
                               _c_int, _c_float, _c_void_p],
     },
     "experts": {
-        "tnx_route": [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p],
+        "tnx_route": [_c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_float,
+                      _c_void_p],
         "tnx_expert_mixture": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                                _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
-                               _c_int, _c_int, _c_void_p],
-        "tnx_gated_activation": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+                               _c_int, _c_int, _c_float, _c_void_p],
+        "tnx_gated_activation": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_float, _c_void_p],
         "tnx_expert_order": [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p,
                              _c_void_p, _c_void_p],
         "tnx_expert_combine": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_void_p],
@@ -160,10 +163,10 @@ _SIGNATURES = {
         "tnx_attention_scored_mfma": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                       _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_void_p, _c_ll,
                                       _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float, _c_int, _c_int, _c_int,
-                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p],
+                                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_int, _c_void_p],
         "tnx_attention_scored": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                                  _c_int, _c_void_p, _c_ll, _c_float, _c_void_p, _c_ll, _c_void_p, _c_int, _c_float,
-                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     },
     "probe": {
         "tnx_probe_stream_read": [_c_void_p, ctypes.c_size_t, _c_void_p, _c_int, _c_void_p],
@@ -1240,8 +1243,11 @@ class HipOps:
                      rotated_pages, across_pages=None):
         """See `ReferenceOps.latent_norms`."""
         t = ctx.num_tokens
-        _want(down, "down", torch.float32, (t, q_rank + kv_rank + rot))
-        _want(q_weight, "query latent norm", torch.float32, (q_rank,))
+        _want(down, "down", torch.float32)
+        if down.dim() != 2 or down.shape[0] != t or down.shape[1] < q_rank + kv_rank + (rot if kv_rank else 0):
+            raise ValueError(f"down must be [{t}, {q_rank + kv_rank + rot} or more], got {tuple(down.shape)}")
+        if q_rank:
+            _want(q_weight, "query latent norm", torch.float32, (q_rank,))
         _want(freqs, "frequencies", torch.float32)
         num_pages = 0
         if kv_rank:
@@ -1249,8 +1255,9 @@ class HipOps:
             num_pages = self._latent_pages(latent_pages, rotated_pages, kv_rank, rot, view.page_size, across_pages)
             _want(view.token_page, "token pages", torch.int32, (t,))
             _want(view.token_offset, "token offsets", torch.int32, (t,))
-        c_q = torch.empty(t, q_rank, dtype=self.dtype, device=down.device)
-        self._call("latent", "tnx_latent_norms", _ptr(down), q_rank, kv_rank, rot, _ptr(q_weight), _ptr(kv_weight),
+        c_q = torch.empty(t, q_rank, dtype=self.dtype, device=down.device) if q_rank else None
+        self._call("latent", "tnx_latent_norms", _ptr(down), down.shape[1], q_rank, kv_rank, rot,
+                   _ptr(q_weight) if q_rank else None, _ptr(kv_weight),
                    float(eps), _ptr(freqs), freqs.numel(), _ptr(ctx.positions), _ptr(view.token_page),
                    _ptr(view.token_offset), _ptr(c_q), _code(self.dtype), _ptr(latent_pages) if kv_rank else None,
                    _ptr(rotated_pages) if kv_rank else None, latent_pages.stride(0) if kv_rank else 0,
@@ -1302,7 +1309,7 @@ class HipOps:
                     and head_size + rot <= 256 and value_size % 16 == 0 and value_size <= 256 and kv_rank % 8 == 0)
 
     def latent_attention_expanded(self, q, w_uk, w_uv, num_heads, head_size, rot, value_size, kv_rank, freqs, scale, ctx,
-                                  view, latent_pages, rotated_pages, window=None):
+                                  view, latent_pages, rotated_pages, window=None, sink=None, gate=None):
         """Attention of a step of prompts' runs with expanded keys and values: `[T, H * value_size]`, what
         `latent_attention` and the product with W_uv give. `w_uk` `[H * head_size, kv_rank]` and `w_uv`
         `[H * value_size, kv_rank]` are the whole matrices."""
@@ -1339,16 +1346,24 @@ class HipOps:
         self._call("latent", "tnx_expanded_attention", _ptr(q), _ptr(k_n), _ptr(r_dense), _ptr(v_t), _ptr(out),
                    _ptr(ctx.run_start), _ptr(ctx.cached_lens), _ptr(start_d), _ptr(base_d), _ptr(ctx.plan["tile_run"]),
                    _ptr(ctx.plan["tile_start"]), tiles, QUERY_TILE, rows, _ptr(freqs), freqs.numel(), float(scale),
-                   num_heads, head_size, rot, value_size, int(window or 0), _stream(),
+                   num_heads, head_size, rot, value_size, int(window or 0), *self._sink_and_gate(sink, gate, t, num_heads),
+                   _stream(),
                    work=(f"{tiles} tiles", rows * num_heads * (head_size + value_size) * 2.0,
                          2.0 * num_heads * (head_size + rot + value_size) * float((lens * seen).sum())))
         return out
+
+    def _sink_and_gate(self, sink, gate, t, num_heads):
+        """(sink pointer, gate pointer, the gate's row distance) for the latent-attention kernels."""
+        if sink is not None:
+            _want(sink, "sinks", torch.float32, (num_heads,))
+        gate_ld = self._rows_apart(gate, "the gate", torch.float32, t, num_heads) if gate is not None else 0
+        return _ptr(sink), _ptr(gate), gate_ld
 
     latent_matrix_unit = True      # tests clear it to run the any-sizes kernel in bfloat16 too
     latent_prompt_kind = 0         # tests set 1: the prompt kernel whose waves each walk the keys for their own queries
 
     def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
-                         rotated_pages, across_pages=None, window=None):
+                         rotated_pages, across_pages=None, window=None, sink=None, gate=None):
         """See `ReferenceOps.latent_attention`. bfloat16 with a latent of a multiple of 16 up to 512 elements, a
         rotated part of a multiple of 8 up to 64 and head sizes in 8s runs on the matrix unit (and reads
         `across_pages`); everything else, and float32, on the kernel for any sizes."""
@@ -1361,6 +1376,7 @@ class HipOps:
         if ctx.max_total > view.width * view.page_size:
             raise ValueError("a request is longer than its block table")
         out = torch.empty(t, num_heads, kv_rank, dtype=self.dtype, device=q.device)
+        finish = self._sink_and_gate(sink, gate, t, num_heads)
         fast = (self.dtype == torch.bfloat16 and self.latent_matrix_unit and across_pages is not None
                 and kv_rank % 16 == 0 and kv_rank <= 512 and rot % 8 == 0 and rot <= 64 and head_size % 8 == 0
                 and "tile_run" in ctx.plan and latent_pages.stride(0) % 8 == 0 and rotated_pages.stride(0) % 8 == 0
@@ -1389,7 +1405,7 @@ class HipOps:
                        _ptr(ctx.plan["decode_runs"]), decodes, _ptr(latent_pages), _ptr(rotated_pages),
                        _ptr(across_pages), latent_pages.stride(0), rotated_pages.stride(0), across_pages.stride(0),
                        _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0),
-                       _ptr(part), splits, per_split, int(self.latent_prompt_kind), _stream(),
+                       _ptr(part), splits, per_split, int(self.latent_prompt_kind), *finish, _stream(),
                        work=(f"{tiles} tiles {decodes} decodes", seen * (2 * kv_rank + rot) * 2,
                              2.0 * num_heads * (2 * kv_rank + rot) * float(
                                  (ctx.run_lens_host * np.minimum(ctx.cached_lens_host + (ctx.run_lens_host + 1) / 2,
@@ -1400,17 +1416,21 @@ class HipOps:
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
                    num_pages, _ptr(latent_pages), _ptr(rotated_pages), latent_pages.stride(0), rotated_pages.stride(0),
                    _ptr(freqs), freqs.numel(), float(scale), num_heads, head_size, rot, kv_rank, int(window or 0), t,
-                   _stream())
+                   *finish, _stream())
         return out
 
 
     # ---------------------------------------------------------------- normed, turned and blended projections
 
     def qkv_prepare(self, proj, num_heads, num_kv, head_size, value_size, cache_head, q_weight, k_weight, eps, freqs,
-                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages, per_head=False):
+                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages, per_head=False,
+                    values_at=None, head_scale=None):
         """See `ReferenceOps.qkv_prepare`. The rows of `proj` may hold more behind the values."""
         t = ctx.num_tokens
-        need = num_heads * head_size + num_kv * (head_size + value_size)
+        need = num_heads * head_size + num_kv * head_size
+        need = max(need, (need if values_at is None else int(values_at)) + num_kv * value_size)
+        if head_scale is not None:
+            _want(head_scale, "head scales", torch.float32, (num_heads,))
         _want(proj, "projections", torch.float32)
         if proj.dim() != 2 or proj.shape[0] != t or proj.shape[1] < need:
             raise ValueError(f"projections must be [{t}, {need} or more], got {tuple(proj.shape)}")
@@ -1437,7 +1457,8 @@ class HipOps:
                    float(scale), _ptr(mix_weight) if first_values is not None else None, _ptr(first_values), first_ld,
                    _ptr(view.token_page), _ptr(view.token_offset), _ptr(q), _ptr(k_pages), _ptr(v_pages),
                    k_pages.stride(0), num_pages, view.page_size, _code(self.dtype), t, num_heads, num_kv, head_size,
-                   value_size, cache_head, int(bool(per_head)), _stream(),
+                   value_size, cache_head, int(bool(per_head)), -1 if values_at is None else int(values_at),
+                   _ptr(head_scale), _stream(),
                    work=(f"{t}x{total}", t * (total * 4 + (num_heads + 2 * num_kv) * cache_head * q.element_size()), 0.0))
         return q
 
@@ -1501,7 +1522,7 @@ class HipOps:
 
     def attention_scored(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None,
                          chunk=None, softcap=None, distance_bias=None, gate=None, value_size=None, out=None,
-                         out_scale=1.0):
+                         out_scale=1.0, gate_per_head=False):
         """See `ReferenceOps.attention_scored`."""
         t = ctx.num_tokens
         value_size = head_size if value_size is None else value_size
@@ -1513,7 +1534,8 @@ class HipOps:
         if out is None:
             out = torch.empty_like(q)
         out_ld = self._rows_apart(out, "the result", self.dtype, t, num_heads * head_size)
-        gate_ld = self._rows_apart(gate, "the gate", torch.float32, t, num_heads * value_size) if gate is not None else 0
+        gate_head = 1 if gate_per_head else value_size
+        gate_ld = self._rows_apart(gate, "the gate", torch.float32, t, num_heads * gate_head) if gate is not None else 0
         far = 0
         if distance_bias is not None:
             _want(distance_bias, "bias by distance", torch.float32)
@@ -1535,7 +1557,7 @@ class HipOps:
                            num_pages, _ptr(tiles), _ptr(ctx.plan["tile_start"]), tiles.numel(), QUERY_TILE, _ptr(out), out_ld,
                            float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far, float(softcap or 0.0),
                            int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size, value_size, sets, pad,
-                           _stream(), work=work)
+                           gate_head, _stream(), work=work)
             if not staged or single.numel():
                 splits, partial = self._scored_splits(ctx, single.numel(), num_heads, num_kv_heads, head_size, window, chunk)
                 self._call("scored", "tnx_attention_scored_mfma", _ptr(q), _ptr(k_pages), _ptr(v_pages), _ptr(ctx.run_start),
@@ -1543,13 +1565,13 @@ class HipOps:
                            _ptr(ctx.plan["tile_start"]), 0 if staged else tiles.numel(), QUERY_TILE, _ptr(single),
                            single.numel(), _ptr(out), out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far,
                            float(softcap or 0.0), int(window or 0), int(chunk or 0), num_heads, num_kv_heads, head_size,
-                           value_size, pad, splits, _ptr(partial), _stream(), work=None if staged else work)
+                           value_size, pad, splits, _ptr(partial), gate_head, _stream(), work=None if staged else work)
             return out
         self._call("scored", "tnx_attention_scored", _ptr(q), _code(self.dtype), _ptr(k_pages), _ptr(v_pages),
                    _ptr(ctx.positions), _ptr(ctx.token_request), _ptr(view.block_table), view.width, view.page_size,
                    num_pages, _ptr(out), out_ld, float(out_scale), _ptr(gate), gate_ld, _ptr(distance_bias), far,
                    float(softcap or 0.0), int(window or 0), int(chunk or 0), t, num_heads, num_kv_heads, head_size,
-                   value_size, pad, _stream(), work=work)
+                   value_size, pad, gate_head, _stream(), work=work)
         return out
 
     scored_decode_splits = None       # tests set it: the blocks that share a decoded token's keys
@@ -1670,7 +1692,7 @@ class HipOps:
 
     # ---------------------------------------------------------------- experts
 
-    def route(self, z, top, score="sigmoid", renormalize=False):
+    def route(self, z, top, score="sigmoid", renormalize=False, correction=None, scale=1.0):
         """See `ReferenceOps.route`."""
         _want(z, "router logits", torch.float32)
         t, experts = z.shape
@@ -1678,11 +1700,13 @@ class HipOps:
             raise ValueError(f"unknown router score {score!r}")
         chosen = torch.empty(t, top, dtype=torch.int32, device=z.device)
         weights = torch.empty(t, top, dtype=torch.float32, device=z.device)
+        if correction is not None:
+            _want(correction, "the choice's correction", torch.float32, (experts,))
         self._call("experts", "tnx_route", _ptr(z), t, experts, top, int(score == "softmax"), int(bool(renormalize)),
-                   _ptr(chosen), _ptr(weights), _stream())
+                   _ptr(chosen), _ptr(weights), _ptr(correction), float(scale), _stream())
         return chosen, weights
 
-    def gated_activation(self, gate_up, activation, row_weights=None):
+    def gated_activation(self, gate_up, activation, row_weights=None, limit=None):
         """See `ReferenceOps.gated_activation`."""
         _want(gate_up, "gate and up", torch.float32)
         t, two_f = gate_up.shape
@@ -1692,7 +1716,7 @@ class HipOps:
             _want(row_weights, "row weights", torch.float32, (t,))
         out = torch.empty(t, two_f // 2, dtype=self.dtype, device=gate_up.device)
         self._call("experts", "tnx_gated_activation", _ptr(gate_up), _ptr(out), _code(self.dtype), t, two_f // 2,
-                   _GATE_ACT[activation], _ptr(row_weights), _stream(),
+                   _GATE_ACT[activation], _ptr(row_weights), float(limit or 0.0), _stream(),
                    work=(f"{t}x{two_f // 2}", t * two_f * 4.0 + out.numel() * out.element_size(), 0.0))
         return out
 
@@ -1704,7 +1728,8 @@ class HipOps:
     expert_row_step = 128
     expert_plain_products = False      # tests set it: the kernel without the matrix unit in bfloat16 too
 
-    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False):
+    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False,
+                       limit=None):
         """See `ReferenceOps.expert_mixture`. `may_wait`: the step is not being recorded, so the host may read
         what the device has made."""
         t, top = chosen.shape
@@ -1747,7 +1772,7 @@ class HipOps:
                     continue
                 b = a + -(-(b - a) // step) * step
                 gu = self.linear(rows[a:b], w_gate_up[e], None, out_f32=True, f32_by_library=True)
-                inner = self.gated_activation(gu, activation, scale[a:b] if on_input else None)
+                inner = self.gated_activation(gu, activation, scale[a:b] if on_input else None, limit=limit)
                 self.linear(inner, w_down[e], None, out_f32=True, f32_by_library=True, into=y[a:b])
             self._call("experts", "tnx_expert_combine", _ptr(y), _ptr(place), None if on_input else _ptr(weights),
                        _ptr(residual), _ptr(out), t, top, width, _stream(),
@@ -1761,7 +1786,7 @@ class HipOps:
         self._call("experts", "tnx_expert_mixture", _ptr(h), _ptr(chosen), _ptr(weights), _ptr(w_gate_up), _ptr(w_down),
                    _ptr(ints[:experts + 1]), _ptr(ints[experts + 1:]), _ptr(inner), _ptr(rows), _ptr(residual), _ptr(out),
                    _code(h.dtype), t, experts, top, width, f, _GATE_ACT[activation], int(weight_on == "input"),
-                   int(bool(self.expert_plain_products)), _stream(),
+                   int(bool(self.expert_plain_products)), float(limit or 0.0), _stream(),
                    work=(f"{t}x{top} of {experts}", used * 3.0 * f * width * item + t * width * (item + 8.0),
                          6.0 * t * top * f * width))
         return out

@@ -127,6 +127,8 @@ class ReferenceOps:
             return 0.5 * y * (1.0 + torch.erf(y / math.sqrt(2.0)))
         if act == "gelu_new":
             return 0.5 * y * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (y + 0.044715 * y * y * y)))
+        if act == "relu2":
+            return torch.relu(y) ** 2
         raise ValueError(f"unknown activation {act!r}")
 
     def linear(self, x, w, bias=None, act=None, residual=None, out_f32=False, f32_by_library=False):
@@ -327,12 +329,13 @@ class ReferenceOps:
         """`down` float32 `[T, q_rank + kv_rank + rot]`: the first q_rank elements, scaled to unit root mean
         square and weighted, come back in the compute dtype; the next kv_rank likewise go to the tokens' places
         in `latent_pages` (and, the page's tokens side by side, in `across_pages` `[pages, kv_rank, page_size]`), the
-        last `rot`, turned by the position, to `rotated_pages` (kv_rank 0: none)."""
+        last `rot`, turned by the position, to `rotated_pages` (kv_rank 0: none). The rows of `down` may hold more
+        behind these; q_rank 0: no query latent, and nothing comes back."""
         x = down.float()
 
         def rms(v, w):
             return v * torch.rsqrt((v * v).mean(-1, keepdim=True) + eps) * w.float()
-        c_q = rms(x[:, :q_rank], q_weight).to(self.dtype)
+        c_q = rms(x[:, :q_rank], q_weight).to(self.dtype) if q_rank else None
         if kv_rank:
             pos = ctx.positions.long()
             page = view.block_table[ctx.token_request.long(), pos // view.page_size].long()
@@ -351,13 +354,28 @@ class ReferenceOps:
         y = torch.einsum("thk,hnk->thn", x.to(w.dtype).float(), w.float()) * alpha
         return (y if out_f32 else y.to(self.dtype)).contiguous()
 
+    @staticmethod
+    def _with_sink(scores, allowed, sink):
+        """Softmax over the allowed keys of `scores` `[H, I, J]`; `sink` `[H]`: the denominator also holds
+        exp(sink) of the head, once."""
+        scores = scores.masked_fill(~allowed.unsqueeze(0), float("-inf"))
+        if sink is None:
+            p = torch.softmax(scores, dim=-1)
+        else:
+            heads, rows, _ = scores.shape
+            beside = sink.float().reshape(heads, 1, 1).expand(heads, rows, 1)
+            p = torch.softmax(torch.cat([scores, beside], dim=-1), dim=-1)[..., :-1]
+        return torch.where(allowed.unsqueeze(0), p, torch.zeros_like(p))
+
     def latent_attention(self, q, q_lat, num_heads, head_size, rot, kv_rank, freqs, scale, ctx, view, latent_pages,
-                         rotated_pages, across_pages=None, window=None):
+                         rotated_pages, across_pages=None, window=None, sink=None, gate=None):
         """For every token and head: scores scale * (q_lat . c[j] + turn(q_r) . k_r[j]) over the cached tokens j
         of its request with j <= position (and position - j < window), softmax, and the weighted sum of the
         c[j]: `[T, H, kv_rank]`. `q` `[T, H * (head_size + rot)]` holds q_r, unturned, behind each head's
         `head_size` elements; `q_lat` is `[T, H, kv_rank]`. `across_pages` hold the c[j] once more, a page's
-        tokens side by side, for kernels that sum from there."""
+        tokens side by side, for kernels that sum from there. `sink` (float32 `[H]`): the softmax's denominator
+        also holds exp(sink) of the head; `gate` (float32 `[T, H]`, rows may lie apart): a head's result is
+        multiplied by sigmoid(gate)."""
         t = q.shape[0]
         ps = view.page_size
         out = torch.empty(t, num_heads, kv_rank, dtype=torch.float32, device=q.device)
@@ -379,12 +397,12 @@ class ReferenceOps:
             allowed = j <= pos
             if window is not None:
                 allowed &= pos - j < window
-            scores = scores.masked_fill(~allowed.unsqueeze(0), float("-inf"))
-            p = torch.softmax(scores, dim=-1)
-            p = torch.where(allowed.unsqueeze(0), p, torch.zeros_like(p))
+            p = self._with_sink(scores, allowed, sink)
             # pages that were given back may hold anything: what the mask hides must not reach the sum
             c = torch.where(torch.isfinite(c), c, torch.zeros_like(c))
             out[s:e] = torch.einsum("hij,jd->ihd", p, c)
+        if gate is not None:
+            out = out * torch.sigmoid(gate.float())[:, :, None]
         return out.to(self.dtype)
 
     expand_prompts = False     # tests set it: steps of prompts' runs alone take `latent_attention_expanded`
@@ -393,7 +411,7 @@ class ReferenceOps:
         return bool(self.expand_prompts and int(ctx.run_lens_host.min()) > 1)
 
     def latent_attention_expanded(self, q, w_uk, w_uv, num_heads, head_size, rot, value_size, kv_rank, freqs, scale, ctx,
-                                  view, latent_pages, rotated_pages, window=None):
+                                  view, latent_pages, rotated_pages, window=None, sink=None, gate=None):
         """Attention with the keys W_uk c and values W_uv c of the cached tokens made explicitly:
         `[T, H * value_size]`, what `latent_attention` and the product with W_uv give by the other order."""
         t, ps = q.shape[0], view.page_size
@@ -417,15 +435,18 @@ class ReferenceOps:
             allowed = j <= pos
             if window is not None:
                 allowed &= pos - j < window
-            p = torch.softmax(scores.masked_fill(~allowed.unsqueeze(0), float("-inf")), dim=-1)
+            p = self._with_sink(scores, allowed, sink)
             out[s:e] = torch.einsum("hij,jhd->ihd", p, val).reshape(e - s, num_heads * value_size)
+        if gate is not None:
+            out = (out.view(t, num_heads, value_size) * torch.sigmoid(gate.float())[:, :, None]).reshape(t, -1)
         return out.to(self.dtype)
 
 
     # ---------------------------------------------------------------- normed, turned and blended projections
 
     def qkv_prepare(self, proj, num_heads, num_kv, head_size, value_size, cache_head, q_weight, k_weight, eps, freqs,
-                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages, per_head=False):
+                    interleaved, scale, mix_weight, first_values, ctx, view, k_pages, v_pages, per_head=False,
+                    values_at=None, head_scale=None):
         """From the float32 projections `proj` `[T, H n + G n + G v]` (bias added) to the queries and the cache:
         the queries and the keys are each scaled to unit root mean square over their whole width and weighted
         (`q_weight`, `k_weight`; None: not), the first `2 len(freqs)` elements of every head are turned by
@@ -433,11 +454,14 @@ class ReferenceOps:
         are multiplied by `scale`, the values become (1 - l) v + l first_values with l = `mix_weight[0]`
         (`first_values` float32 `[T, G v]`, a view whose rows may lie apart; None: not). Keys and values go to their
         tokens' places in the pages, heads filled up with zeros to `cache_head` elements; the queries come back
-        `[T, H cache_head]`, filled up alike, in the compute dtype."""
+        `[T, H cache_head]`, filled up alike, in the compute dtype. `values_at`: the column of a row where the
+        values begin, if not behind the keys (the keys' own first column: the values are the keys as projected).
+        `head_scale` (float32 `[H]`): a query head's elements are multiplied by its number as well."""
         t = proj.shape[0]
         nq, nk, nv = num_heads * head_size, num_kv * head_size, num_kv * value_size
         x = proj.float()
-        q, k, v = x[:, :nq], x[:, nq:nq + nk], x[:, nq + nk:nq + nk + nv]
+        at = nq + nk if values_at is None else int(values_at)
+        q, k, v = x[:, :nq], x[:, nq:nq + nk], x[:, at:at + nv]
         if per_head:
             # every head to unit root mean square by itself; the weights, if any, are still one a projection element
             q, k = q.reshape(t, num_heads, head_size), k.reshape(t, num_kv, head_size)
@@ -476,18 +500,21 @@ class ReferenceOps:
         v_pages[page, :, :, off] = 0
         v_pages[page, :, :value_size, off] = v.to(v_pages.dtype)
         out = torch.zeros(t, num_heads, cache_head, dtype=self.dtype, device=proj.device)
+        if head_scale is not None:
+            q = q * head_scale.float()[None, :, None]
         out[:, :, :head_size] = (q * scale).to(self.dtype)
         return out.reshape(t, num_heads * cache_head)
 
     def attention_scored(self, q, num_heads, num_kv_heads, head_size, ctx, view, k_pages, v_pages, window=None,
                          chunk=None, softcap=None, distance_bias=None, gate=None, value_size=None, out=None,
-                         out_scale=1.0):
+                         out_scale=1.0, gate_per_head=False):
         """Attention whose scores or mask are not the plain ones. For a query at position i and a key at j <= i of
         its request: s = q . k (the query comes scaled); with `softcap` c, s <- c tanh(s / c); with
         `distance_bias` (float32 `[heads, D + 1]`), s <- s + distance_bias[head, min(i - j, D)]. Visible are the
         keys with i - j < window (if given) and floor(j / chunk) = floor(i / chunk) (if given). Softmax over the
         visible keys, times the values. `gate` (float32 `[T, heads * value_size]`, rows may lie apart): the first
-        `value_size` elements of every head are multiplied by sigmoid(gate). The result times `out_scale` goes to
+        `value_size` elements of every head are multiplied by sigmoid(gate) (`gate_per_head`: `[T, heads]`, one
+        number for all elements of a head). The result times `out_scale` goes to
         `out` (`[T, heads * head_size]` in the compute dtype, rows may lie apart) or to a new tensor."""
         t = q.shape[0]
         value_size = head_size if value_size is None else value_size
@@ -526,7 +553,7 @@ class ReferenceOps:
             p = torch.softmax(scores, dim=-1)
             res[s:e] = (p @ vals.transpose(1, 2)).permute(1, 0, 2)
         if gate is not None:
-            res[:, :, :value_size] *= torch.sigmoid(gate.float()).reshape(t, num_heads, value_size)
+            res[:, :, :value_size] *= torch.sigmoid(gate.float()).reshape(t, num_heads, 1 if gate_per_head else value_size)
         res = (res * out_scale).reshape(t, num_heads * head_size)
         if out is None:
             return res.to(self.dtype)
@@ -669,34 +696,45 @@ class ReferenceOps:
 
     # ---------------------------------------------------------------- experts
 
-    def route(self, z, top, score="sigmoid", renormalize=False):
+    def route(self, z, top, score="sigmoid", renormalize=False, correction=None, scale=1.0):
         """float32 router logits `[T, E]` -> (int32 `[T, top]` the experts with the largest scores, the lower
         number first where two are equal; float32 `[T, top]` their scores, sigmoid(z) or softmax(z), divided by
         their sum with `renormalize`). The ranking is by the logits, which both scores grow with: two large
-        logits that float32 still tells apart can have scores that it does not."""
+        logits that float32 still tells apart can have scores that it does not. With `correction` (float32 `[E]`)
+        the ranking is by score + correction, and the weights are the scores without it; `scale` multiplies the
+        weights."""
         s = torch.sigmoid(z.float()) if score == "sigmoid" else torch.softmax(z.float(), dim=-1)
-        order = torch.sort(z.float(), dim=-1, descending=True, stable=True).indices[:, :top]
+        ranked = z.float() if correction is None else s + correction.float()
+        order = torch.sort(ranked, dim=-1, descending=True, stable=True).indices[:, :top]
         w = torch.gather(s, 1, order)
         if renormalize:
             w = w / w.sum(-1, keepdim=True)
+        if scale != 1.0:
+            w = w * scale
         return order.to(torch.int32).contiguous(), w.contiguous()
 
     @staticmethod
-    def _gate(g, activation):
+    def _gated(g, u, activation, limit=None):
+        """What a gated expert makes of its two halves: act(g) * u; "clamped_swiglu": with g' = min(g, limit) and
+        u' = clamp(u, -limit, limit), g' sigmoid(1.702 g') (u' + 1)."""
+        if activation == "clamped_swiglu":
+            g, u = g.clamp(max=limit), u.clamp(min=-limit, max=limit)
+            return g * torch.sigmoid(1.702 * g) * (u + 1.0)
         if activation == "silu":
-            return g * torch.sigmoid(g)
-        return ReferenceOps.activation(g, activation)
+            return g * torch.sigmoid(g) * u
+        return ReferenceOps.activation(g, activation) * u
 
-    def gated_activation(self, gate_up, activation, row_weights=None):
+    def gated_activation(self, gate_up, activation, row_weights=None, limit=None):
         """`act(g) * u` from float32 `[T, 2 F]` = [g | u], in the compute dtype; `row_weights` `[T]`: a factor a
         row on both g and u."""
         f = gate_up.shape[1] // 2
         g, u = gate_up[:, :f].float(), gate_up[:, f:].float()
         if row_weights is not None:
             g, u = g * row_weights.float()[:, None], u * row_weights.float()[:, None]
-        return (self._gate(g, activation) * u).to(self.dtype)
+        return self._gated(g, u, activation, limit).to(self.dtype)
 
-    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False):
+    def expert_mixture(self, h, chosen, weights, w_gate_up, w_down, activation, weight_on, residual=None, may_wait=False,
+                       limit=None):
         """float32 `residual + sum_c expert_(chosen[t, c])(h[t])` with the weights `weights[t, c]` on the expert's
         input (`weight_on="input"`: act(w g) * (w u), the float32 sums of the first product times w) or on its
         output. `w_gate_up` `[E, 2 F, D]` (gate rows, then up rows), `w_down` `[E, D, F]`."""
@@ -711,7 +749,7 @@ class ReferenceOps:
             w = weights[:, c].float()[:, None]
             if weight_on == "input":
                 gu = gu * w
-            inner = (self._gate(gu[:, :f], activation) * gu[:, f:]).to(self.dtype)
+            inner = self._gated(gu[:, :f], gu[:, f:], activation, limit).to(self.dtype)
             y = torch.einsum("tf,tdf->td", inner.to(w_down.dtype).float(), w_down[e].float())
             out = out + (y if weight_on == "input" else y * w)
         return out

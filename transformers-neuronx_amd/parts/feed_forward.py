@@ -19,7 +19,8 @@ class DenseFeedForward(FeedForward):
 
         `activation="poly_norm"` is no function of one element: with N(v) = v / sqrt(mean(v^2) + eps) over a
         token's inner values, act(z) = a N(z) + b N(z^2) + c N(z^3) + e, powers element by element, the four
-        numbers being the tensor `act_name`. Sums and roots are float32."""
+        numbers being the tensor `act_name`. Sums and roots are float32. `activation="relu2"` is the square of
+        relu."""
         self.width, self.inner, self.activation, self.has_bias = width, inner, activation, bias
         self.up_name, self.down_name, self.weight_suffix = up_name, down_name, weight_suffix
         self.act_name, self.eps = act_name, float(eps)
@@ -114,19 +115,36 @@ class ExpertMixture(FeedForward):
     scores, divided by their sum with `renormalize`. An expert is W_down (act(W_gate x) * (W_up x)), no biases.
     `weight_on="input"`: the result is the sum of expert(w h), the weight applied to what the expert reads;
     `"output"`: the sum of w expert(h). The shared expert (`shared_inner` > 0) is of the same form, reads h and
-    is added. The weights enter the float32 sums of the first products, so nothing is rounded twice."""
+    is added. The weights enter the float32 sums of the first products, so nothing is rounded twice.
+
+    `correction_name`: a tensor of one number an expert that is added to the scores where the experts are chosen
+    and nowhere else (the weights are the scores without it). `route_scale`: the weights times this number.
+    `activation="clamped_swiglu"` with `limit` (`shared_limit` for the shared expert): g = min(W_gate x, limit),
+    u = clamp(W_up x, -limit, limit), and the expert is W_down (g sigmoid(1.702 g) (u + 1))."""
 
     recordable = True
 
     def __init__(self, width: int, experts: int, top: int, inner: int, router_name: str, expert_name: str, names,
                  shared_inner: int = 0, shared_name: str = "shared.", score: str = "sigmoid", renormalize: bool = False,
-                 weight_on: str = "output", activation: str = "silu", weight_suffix: str = ""):
+                 weight_on: str = "output", activation: str = "silu", weight_suffix: str = "",
+                 correction_name: str = None, route_scale: float = 1.0, limit: float = None, shared_limit: float = None):
         """`expert_name`: a format string that takes the expert's number ("e{}."); `names`: the names of an
         expert's gate, up and down matrices."""
         if not 1 <= top <= experts:
             raise ValueError(f"a token takes {top} of {experts} experts")
-        if score not in ("sigmoid", "softmax") or weight_on not in ("input", "output") or activation not in ("silu", "gelu_new"):
+        if score not in ("sigmoid", "softmax") or weight_on not in ("input", "output") \
+                or activation not in ("silu", "gelu_new", "clamped_swiglu"):
             raise ValueError(f"mixture: score {score!r}, weight_on {weight_on!r}, activation {activation!r}")
+        if activation == "clamped_swiglu":
+            if limit is None or not float(limit) > 0 or (shared_inner and not float(shared_limit or 0) > 0):
+                raise ValueError("mixture: activation 'clamped_swiglu' needs a positive `limit` (and `shared_limit`)")
+            if weight_on != "output":
+                raise ValueError("mixture: a clamped expert takes its weight on the output")
+        if correction_name and (score != "sigmoid" or renormalize):
+            raise ValueError("mixture: a correction of the choice goes with sigmoid scores that are not renormalized")
+        self.correction_name, self.route_scale = correction_name, float(route_scale)
+        self.limit = float(limit) if limit is not None else None
+        self.shared_limit = float(shared_limit) if shared_limit is not None else None
         self.width, self.experts, self.top, self.inner, self.shared_inner = width, experts, top, inner, shared_inner
         self.router_name, self.expert_name, self.shared_name = router_name, expert_name, shared_name
         self.names, self.weight_suffix = tuple(names), weight_suffix
@@ -143,6 +161,8 @@ class ExpertMixture(FeedForward):
         for e in range(self.experts):
             d += self._expert_decls(prefix + self.expert_name.format(e), self.inner)
         d.append(ParamDecl(f"{prefix}{self.router_name}{self.weight_suffix}", (self.experts, self.width)))
+        if self.correction_name:
+            d.append(ParamDecl(f"{prefix}{self.correction_name}", (self.experts,), "vector"))
         if self.shared_inner:
             d += self._expert_decls(prefix + self.shared_name, self.shared_inner)
         return d
@@ -157,6 +177,7 @@ class ExpertMixture(FeedForward):
         self.w_gate_up = torch.stack([torch.cat([tensors[f"{p}{g}{s}"], tensors[f"{p}{u}{s}"]], dim=0) for p in each]).contiguous()
         self.w_down = torch.stack([tensors[f"{p}{d}{s}"] for p in each]).contiguous()
         self.w_router = ops.prepare_weight(tensors[f"{prefix}{self.router_name}{s}"])
+        self.correction = tensors[f"{prefix}{self.correction_name}"] if self.correction_name else None
         if self.shared_inner:
             p = prefix + self.shared_name
             self.w_shared_in = ops.prepare_weight(torch.cat([tensors[f"{p}{g}{s}"], tensors[f"{p}{u}{s}"]], dim=0).contiguous())
@@ -168,12 +189,17 @@ class ExpertMixture(FeedForward):
     def forward(self, h, ctx, residual):
         ops = self.ops
         z = ops.linear(h, self.w_router, None, out_f32=True, f32_by_library=True)
-        chosen, weights = ops.route(z, self.top, self.score, self.renormalize)
+        more = {}
+        if self.correction is not None or self.route_scale != 1.0:
+            more = dict(correction=self.correction, scale=self.route_scale)
+        chosen, weights = ops.route(z, self.top, self.score, self.renormalize, **more)
+        limit = dict(limit=self.limit) if self.limit is not None else {}
         # (a step that is being recorded is sized by `length_bound`; any other may let the host read)
         x = ops.expert_mixture(h, chosen, weights, self.w_gate_up, self.w_down, self.activation, self.weight_on, residual,
-                               may_wait=ctx is not None and ctx.length_bound is None)
+                               may_wait=ctx is not None and ctx.length_bound is None, **limit)
         if not self.shared_inner:
             return x
+        limit = dict(limit=self.shared_limit) if self.shared_limit is not None else {}
         inner = ops.gated_activation(ops.linear(h, self.w_shared_in, None, out_f32=True, f32_by_library=True),
-                                     self.activation)
+                                     self.activation, **limit)
         return ops.linear(inner, self.w_shared_down, None, residual=x, out_f32=True)

@@ -57,7 +57,8 @@ class Attention(Mixer):
                  own_kv: bool = True, rotation=None, value_size: Optional[int] = None, out_bias: Optional[bool] = None,
                  qk_norm=None, value_mix=None, weight_suffix: str = ".weight", bias_suffix: str = ".bias",
                  softcap: Optional[float] = None, distance_bias=None, chunk: Optional[int] = None,
-                 out_gate: Optional[str] = None):
+                 out_gate: Optional[str] = None, out_gate_per_head: bool = False, values_from_keys: bool = False,
+                 head_scale: Optional[str] = None):
         """`names`: the checkpoint's names of the query, key, value and output projections, relative to
         the mixer's prefix (the architecture's spec gives them); a matrix's name adds `weight_suffix`, a bias's
         `bias_suffix`. `out_bias`: whether the output projection has a bias (as the others, if not said).
@@ -85,7 +86,13 @@ class Attention(Mixer):
         query at position i sees the keys j <= i with floor(j / m) = floor(i / m), positions counted from the
         request's start. `out_gate`: the name of a matrix W_g `[heads * value_size, width]`; the heads' results
         side by side are multiplied by sigmoid(W_g h) before the output projection (the gate's rows ride in the
-        one input projection)."""
+        one input projection); with `out_gate_per_head` W_g is `[heads, width]` and a head's whole result is
+        multiplied by its one number.
+
+        `values_from_keys`: there is no value projection (its name in `names` is not read): a token's values are
+        its keys as projected, before their norm and turn. `head_scale`: the name of a tensor of one number a query
+        head that multiplies the head's scores (beside `scale`). With `shared` in `qk_norm` (which implies
+        `per_head`) the two weight tensors hold one head's `head_size` elements, the same for every head."""
         self.width, self.num_heads, self.head_size = width, num_heads, head_size
         self.num_kv_heads = num_kv_heads if num_kv_heads is not None else num_heads
         if self.num_heads % self.num_kv_heads:
@@ -98,11 +105,19 @@ class Attention(Mixer):
         self.softcap = float(softcap) if softcap else None
         self.distance_bias = dict(distance_bias) if distance_bias else None
         self.chunk = int(chunk) if chunk else None
-        self.out_gate = out_gate
+        self.out_gate, self.out_gate_per_head = out_gate, bool(out_gate_per_head) and bool(out_gate)
+        self.values_from_keys, self.head_scale = bool(values_from_keys), head_scale
+        if self.qk_norm and self.qk_norm.get("shared"):
+            self.qk_norm["per_head"] = True
+        if self.values_from_keys and self.value_size != head_size:
+            raise ValueError(f"values that are the keys have the keys' size ({head_size}), not {self.value_size}")
+        if self.values_from_keys and self.value_mix:
+            raise ValueError("values that are the keys are not blended")
         if self.chunk is not None and window is not None:
             raise ValueError("an attention mixer masks by a window or by chunks, not both")
         self.scored = bool(self.softcap or self.distance_bias or self.chunk or out_gate)
-        self.prepared = bool(self.qk_norm or self.value_mix or halves or self.value_size != head_size or self.scored)
+        self.prepared = bool(self.qk_norm or self.value_mix or halves or self.value_size != head_size or self.scored
+                             or self.values_from_keys or head_scale)
         self.defer_out = False      # set by a mixer that runs this one beside another and owns the output product
         if self.prepared:
             if not own_kv:
@@ -133,7 +148,7 @@ class Attention(Mixer):
         q_out = self.num_heads * self.head_size
         kv_out = self.num_kv_heads * self.head_size
         v_out = self.num_kv_heads * self.value_size
-        outs = [(qn, q_out)] + ([(kn, kv_out), (vn, v_out)] if self.own_kv else [])
+        outs = [(qn, q_out)] + ([(kn, kv_out)] + ([] if self.values_from_keys else [(vn, v_out)]) if self.own_kv else [])
         d = []
         for n, out in outs:
             d.append(ParamDecl(f"{prefix}{n}{ws}", (out, self.width)))
@@ -143,13 +158,17 @@ class Attention(Mixer):
         if self.has_out_bias:
             d.append(ParamDecl(f"{prefix}{on}{bs}", (self.width,), "vector"))
         if self.qk_norm and self.qk_norm.get("weighted", True):
-            d += [ParamDecl(f"{prefix}{qn}{self.qk_norm['suffix']}", (q_out,), "vector", "around_one"),
-                  ParamDecl(f"{prefix}{kn}{self.qk_norm['suffix']}", (kv_out,), "vector", "around_one")]
+            shared = self.qk_norm.get("shared")
+            d += [ParamDecl(f"{prefix}{qn}{self.qk_norm['suffix']}", (self.head_size if shared else q_out,), "vector", "around_one"),
+                  ParamDecl(f"{prefix}{kn}{self.qk_norm['suffix']}", (self.head_size if shared else kv_out,), "vector", "around_one")]
+        if self.head_scale:
+            d.append(ParamDecl(f"{prefix}{self.head_scale}", (self.num_heads,), "vector", "around_one"))
         if self.distance_bias:
             d.append(ParamDecl(f"{prefix}{self.distance_bias['name']}", (self.distance_bias.get("rows"), self.num_heads),
                                "vector"))
         if self.out_gate:
-            d.append(ParamDecl(f"{prefix}{self.out_gate}{ws}", (self.num_heads * self.value_size, self.width)))
+            d.append(ParamDecl(f"{prefix}{self.out_gate}{ws}",
+                               (self.num_heads * (1 if self.out_gate_per_head else self.value_size), self.width)))
         if self.value_mix and not self.value_mix["first"]:
             d.append(ParamDecl(f"{prefix}{self.value_mix['name']}", (), "vector", "around_half"))
         if self.rotation is not None:
@@ -160,7 +179,8 @@ class Attention(Mixer):
         super().load(tensors, prefix, ops, dtype)
         qn, kn, vn, on = self.names
         ws, bs = self.weight_suffix, self.bias_suffix
-        ins = [qn] + ([kn, vn] if self.own_kv else []) + ([self.out_gate] if self.out_gate else [])
+        ins = ([qn] + ([kn] + ([] if self.values_from_keys else [vn]) if self.own_kv else [])
+               + ([self.out_gate] if self.out_gate else []))
         # One fused projection: a plain concatenation of the rows (the reference's
         # fused form interleaves per tensor-parallel shard, utils.py:189-242).
         self.w_qkv = ops.prepare_weight(torch.cat([tensors[f"{prefix}{n}{ws}"] for n in ins], dim=0).contiguous())
@@ -192,6 +212,10 @@ class Attention(Mixer):
         if self.qk_norm and self.qk_norm.get("weighted", True):
             self.q_norm = tensors[f"{prefix}{qn}{self.qk_norm['suffix']}"]
             self.k_norm = tensors[f"{prefix}{kn}{self.qk_norm['suffix']}"]
+            if self.qk_norm.get("shared"):      # one head's weights, the same for every head: spread once
+                self.q_norm = self.q_norm.repeat(self.num_heads).contiguous()
+                self.k_norm = self.k_norm.repeat(self.num_kv_heads).contiguous()
+        self.head_scales = tensors[f"{prefix}{self.head_scale}"] if self.head_scale else None
         if self.value_mix and not self.value_mix["first"]:
             self.mix_weight = tensors[f"{prefix}{self.value_mix['name']}"].reshape(1)
 
@@ -250,22 +274,29 @@ class Attention(Mixer):
                 if first is None:
                     raise ValueError("a layer blends its values with those of a layer that has not run in this pass")
         rot = self.rotation
+        more = {"per_head": True} if (self.qk_norm or {}).get("per_head") else {}
+        if self.values_from_keys:
+            more["values_at"] = self.num_heads * self.head_size        # the keys' columns are read a second time
+        if self.head_scales is not None:
+            more["head_scale"] = self.head_scales
         q = ops.qkv_prepare(proj, self.num_heads, self.num_kv_heads, self.head_size, self.value_size, self.cache_head,
                             self.q_norm, self.k_norm, self.qk_norm["eps"] if self.qk_norm else 0.0, self.freqs,
                             bool(rot.interleaved) if rot is not None else False, self.scale, self.mix_weight, first,
-                            ctx, view, cache.k_pages, cache.v_pages,
-                            **({"per_head": True} if (self.qk_norm or {}).get("per_head") else {}))
+                            ctx, view, cache.k_pages, cache.v_pages, **more)
         if not self.scored and out is None:
             return ops.attention(q, self.num_heads, self.num_kv_heads, self.cache_head, ctx, view, cache.k_pages,
                                  cache.v_pages, self.window)
-        gate = None
+        gate, more = None, {}
         if self.out_gate:
-            at = self.num_heads * self.head_size + self.num_kv_heads * (self.head_size + self.value_size)
-            gate = proj[:, at:at + self.num_heads * self.value_size]
+            at = self.num_heads * self.head_size + self.num_kv_heads * (
+                self.head_size + (0 if self.values_from_keys else self.value_size))
+            gate = proj[:, at:at + self.num_heads * (1 if self.out_gate_per_head else self.value_size)]
+            if self.out_gate_per_head:
+                more["gate_per_head"] = True
         return ops.attention_scored(q, self.num_heads, self.num_kv_heads, self.cache_head, ctx, view, cache.k_pages,
                                     cache.v_pages, window=self.window, chunk=self.chunk, softcap=self.softcap,
                                     distance_bias=self.bias_by_distance, gate=gate, value_size=self.value_size,
-                                    out=out, out_scale=out_scale)
+                                    out=out, out_scale=out_scale, **more)
 
     def forward(self, h, ctx, cache, residual):
         if cache.writes != self.own_kv:
@@ -313,6 +344,14 @@ class LatentAttention(Mixer):
     other (`ops.latent_expands`): the keys W_uk c and values W_uv c of what the runs can see are made once for
     the step, and a (query, key) pair costs 2 (n + r + v) multiply-adds a head instead of 2 (2R + r).
 
+    `q_rank=None`: no query latent: q = W_q h, one matrix (the second of `names`; the first is not read).
+    `sink`: the name of a tensor of one number a head; the softmax's denominator also holds exp(sink), once, with no
+    key and no value behind it. `out_gate`: the name of a matrix W_g `[heads, width]`; a head's result is multiplied
+    by sigmoid(W_g h) of that head before W_o (its rows ride in the product with W_dkv). A rotation that pairs
+    element i with i + dims / 2 is brought to neighbouring pairs by putting the rows of the matrices that make
+    q_r and k_r in the order (0, dims/2, 1, dims/2 + 1, ...) once, at load: q_r and k_r meet in a dot product
+    only, which does not see the order.
+
     `own_kv=False`: no W_dkv; the mixer reads the cache of another call of the run order, whose R, r and
     rotation are its own. `keep`: the tokens the cache keeps: a number, "all", or None for the mixer's own window;
     a cache that is read by mixers of different windows keeps the most any of them sees.
@@ -321,8 +360,9 @@ class LatentAttention(Mixer):
     recordable = True
 
     def __init__(self, width: int, num_heads: int, head_size: int, rot_size: int, value_size: int, kv_rank: int,
-                 q_rank: int, scale: float, eps: float, rotation, names, window: Optional[int] = None,
-                 keep=None, own_kv: bool = True, norm_suffix: str = ".norm", weight_suffix: str = ""):
+                 q_rank: Optional[int], scale: float, eps: float, rotation, names, window: Optional[int] = None,
+                 keep=None, own_kv: bool = True, norm_suffix: str = ".norm", weight_suffix: str = "",
+                 sink: Optional[str] = None, out_gate: Optional[str] = None):
         """`names`: the checkpoint's names, relative to the mixer's prefix, of W_dq, W_uq, W_dkv, W_uk, W_uv and
         W_o; a latent's norm weight is its down-projection's name with `norm_suffix`."""
         self.width, self.num_heads, self.head_size, self.rot_size = width, num_heads, head_size, rot_size
@@ -337,6 +377,9 @@ class LatentAttention(Mixer):
         if len(self.names) != 6:
             raise ValueError("names: W_dq, W_uq, W_dkv, W_uk, W_uv, W_o, six names")
         self.norm_suffix, self.weight_suffix = norm_suffix, weight_suffix
+        self.sink, self.out_gate = sink, out_gate
+        if out_gate and not own_kv:
+            raise ValueError("a latent-attention mixer with a gate on its heads makes its own latents")
         self.rotation = POSITIONS.build(rotation)
         if rot_size % 2 or self.rotation.dims > rot_size:
             raise ValueError(f"the rotated part has {rot_size} elements; the rotation turns {self.rotation.dims}")
@@ -352,11 +395,18 @@ class LatentAttention(Mixer):
         return {"attention": attention_plan}
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
-        dq, uq, dkv, uk, uv, o = (prefix + n for n in self.names)
+        dq, uq, dkv, uk, uv, o = (prefix + (n or "") for n in self.names)
         s, h = self.weight_suffix, self.num_heads
-        d = [ParamDecl(dq + s, (self.q_rank, self.width)),
-             ParamDecl(dq + self.norm_suffix, (self.q_rank,), "vector", "around_one"),
-             ParamDecl(uq + s, (h * (self.head_size + self.rot_size), self.q_rank))]
+        if self.q_rank is None:
+            d = [ParamDecl(uq + s, (h * (self.head_size + self.rot_size), self.width))]
+        else:
+            d = [ParamDecl(dq + s, (self.q_rank, self.width)),
+                 ParamDecl(dq + self.norm_suffix, (self.q_rank,), "vector", "around_one"),
+                 ParamDecl(uq + s, (h * (self.head_size + self.rot_size), self.q_rank))]
+        if self.sink:
+            d.append(ParamDecl(prefix + self.sink, (h,), "vector"))
+        if self.out_gate:
+            d.append(ParamDecl(prefix + self.out_gate + s, (h, self.width)))
         if self.own_kv:
             d += [ParamDecl(dkv + s, (self.kv_rank + self.rot_size, self.width)),
                   ParamDecl(dkv + self.norm_suffix, (self.kv_rank,), "vector", "around_one")]
@@ -367,14 +417,32 @@ class LatentAttention(Mixer):
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
-        dq, uq, dkv, uk, uv, o = (prefix + n for n in self.names)
+        dq, uq, dkv, uk, uv, o = (prefix + (n or "") for n in self.names)
         s, h = self.weight_suffix, self.num_heads
-        # one product for both latents: the rows of W_dq, then those of W_dkv
-        down = [tensors[dq + s]] + ([tensors[dkv + s]] if self.own_kv else [])
+        self.rotation.load(tensors, prefix + "rotation", ops, dtype)
+        self.freqs = self.rotation.frequencies()
+        n, r, dims = self.head_size, self.rot_size, self.rotation.dims
+        w_uq, w_dkv = tensors[uq + s], (tensors[dkv + s] if self.own_kv else None)
+        if not self.rotation.interleaved:
+            if not self.own_kv:
+                raise ValueError("a rotation by halves is brought to neighbouring pairs in the matrices that make "
+                                 "both q_r and k_r: the mixer must own the latter")
+            # element i and element i + dims / 2 of the rotated part become neighbours
+            order = torch.arange(r, device=w_uq.device)
+            order[:dims] = torch.stack([torch.arange(dims // 2), torch.arange(dims // 2) + dims // 2], dim=1).reshape(-1) \
+                .to(w_uq.device)
+            rows = (torch.arange(h, device=w_uq.device)[:, None] * (n + r) + n + order[None, :]).reshape(-1)
+            w_uq = w_uq.clone()
+            w_uq.view(h, n + r, -1)[:, n:] = tensors[uq + s][rows].view(h, r, -1)
+            w_dkv = torch.cat([w_dkv[:self.kv_rank], w_dkv[self.kv_rank + order]], dim=0)
+        # one product for what is wanted in float32: the rows of W_dq, then those of W_dkv, then the gate's
+        down = (([tensors[dq + s]] if self.q_rank is not None else []) + ([w_dkv] if self.own_kv else [])
+                + ([tensors[prefix + self.out_gate + s]] if self.out_gate else []))
         self.w_down = ops.prepare_weight(torch.cat(down, dim=0).contiguous())
-        self.q_norm = tensors[dq + self.norm_suffix]
+        self.q_norm = tensors[dq + self.norm_suffix] if self.q_rank is not None else None
         self.kv_norm = tensors[dkv + self.norm_suffix] if self.own_kv else None
-        self.w_uq = ops.prepare_weight(tensors[uq + s])
+        self.sinks = tensors[prefix + self.sink] if self.sink else None
+        self.w_uq = ops.prepare_weight(w_uq.contiguous())
         # W_uk a head, transposed: [H, R, n], the matrix that takes a head's q_n to its q_lat
         self.w_uk_t = tensors[uk + s].view(h, self.head_size, self.kv_rank).transpose(1, 2).contiguous()
         self.w_uv = tensors[uv + s].view(h, self.value_size, self.kv_rank).contiguous()
@@ -382,10 +450,6 @@ class LatentAttention(Mixer):
         self.w_uk_whole = ops.prepare_weight(tensors[uk + s])
         self.w_uv_whole = tensors[uv + s]
         self.w_o = ops.prepare_weight(tensors[o + s])
-        self.rotation.load(tensors, prefix + "rotation", ops, dtype)
-        self.freqs = self.rotation.frequencies()
-        if not self.rotation.interleaved:
-            raise ValueError("latent attention turns neighbouring pairs (the interleaved layout)")
 
     def first_weight(self):
         return None          # the product's float32 result goes to two norms: the norm before it stays a kernel
@@ -404,18 +468,25 @@ class LatentAttention(Mixer):
             raise ValueError(f"the cache holds latents of {latent.shape[-1]} + {rotated.shape[-1]} elements, "
                              f"this mixer reads {self.kv_rank} + {r}")
         down = ops.linear(h, self.w_down, None, out_f32=True, f32_by_library=True)
-        c_q = ops.latent_norms(down, self.q_rank, self.kv_rank if self.own_kv else 0, r if self.own_kv else 0,
+        q_rank = self.q_rank or 0
+        c_q = ops.latent_norms(down, q_rank, self.kv_rank if self.own_kv else 0, r if self.own_kv else 0,
                                self.q_norm, self.kv_norm, self.eps, self.freqs, ctx, view, latent, rotated, across)
-        q = ops.linear(c_q, self.w_uq, None)
+        q = ops.linear(c_q if self.q_rank is not None else h, self.w_uq, None)
+        more = {}
+        if self.sinks is not None:
+            more["sink"] = self.sinks
+        if self.out_gate:
+            at = q_rank + self.kv_rank + r
+            more["gate"] = down[:, at:at + heads]
         if ops.latent_expands(ctx, n, r, self.value_size, self.kv_rank):
             # a step of prompts' runs alone: keys and values made from the latents, attention on them
             values = ops.latent_attention_expanded(q, self.w_uk_whole, self.w_uv_whole, heads, n, r, self.value_size,
                                                    self.kv_rank, self.freqs, self.scale, ctx, view, latent, rotated,
-                                                   self.window)
+                                                   self.window, **more)
             return ops.linear(values, self.w_o, None, residual=residual, out_f32=True, f32_by_library=residual is None)
         q_lat = ops.batched_linear(q.view(-1, heads, n + r)[:, :, :n], self.w_uk_t)
         o_lat = ops.latent_attention(q, q_lat, heads, n, r, self.kv_rank, self.freqs, self.scale, ctx, view,
-                                     latent, rotated, across, self.window)
+                                     latent, rotated, across, self.window, **more)
         values = ops.batched_linear(o_lat, self.w_uv)
         return ops.linear(values.view(-1, heads * self.value_size), self.w_o, None, residual=residual, out_f32=True,
                           f32_by_library=residual is None)

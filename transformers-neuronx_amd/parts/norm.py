@@ -62,18 +62,23 @@ class RMSNorm(Norm):
 
     recordable = True
 
-    def __init__(self, width: int, eps: float, weight_suffix: str = ".weight", unit_offset: bool = False):
+    def __init__(self, width: int, eps: float, weight_suffix: str = ".weight", unit_offset: bool = False,
+                 scalar: bool = False):
+        """`scalar`: the checkpoint's weight is one number (a tensor without dimensions) that multiplies every
+        coordinate; it is spread over the width once, at load."""
         self.width, self.eps, self.weight_suffix = width, float(eps), weight_suffix
-        self.unit_offset = bool(unit_offset)
+        self.unit_offset, self.scalar = bool(unit_offset), bool(scalar)
         self.weight = None
 
     def param_decls(self, prefix: str) -> List[ParamDecl]:
-        return [ParamDecl(prefix + self.weight_suffix, (self.width,), "vector",
+        return [ParamDecl(prefix + self.weight_suffix, () if self.scalar else (self.width,), "vector",
                           "normal" if self.unit_offset else "around_one")]
 
     def load(self, tensors: Dict, prefix: str, ops, dtype) -> None:
         super().load(tensors, prefix, ops, dtype)
         self.weight = tensors[prefix + self.weight_suffix]
+        if self.scalar:
+            self.weight = self.weight.reshape(1).expand(self.width).contiguous()
         if self.unit_offset:
             self.weight = (self.weight.float() + 1.0).contiguous()
 

@@ -77,7 +77,8 @@ class RotaryPositions(PositionEncoding):
     `scaling` = {factor, low, high, original} stretches the slow turns for requests longer than `original`
     tokens: a frequency f with wavelength l = 2 pi / f is kept where l < original / high, becomes f / factor
     where l > original / low, and between the two (1 - s) f / factor + s f with
-    s = (original / l - low) / (high - low).
+    s = (original / l - low) / (high - low). `scaling` = {factor} alone divides every frequency by the factor
+    (positions stretched linearly).
 
     Two ways to use it: `pair_tables` (the attention mixer's pairwise form, for `max_positions` positions,
     interleaved pairs only), or `frequencies()`, for a mixer whose kernels make the angles themselves."""
@@ -89,7 +90,11 @@ class RotaryPositions(PositionEncoding):
             raise ValueError(f"rotary positions turn pairs: dims must be even, got {dims}")
         self.base, self.dims, self.max_positions, self.interleaved = float(base), dims, max_positions, interleaved
         self.scaling = dict(scaling) if scaling else None
-        if self.scaling:
+        self.linear_scaling = bool(self.scaling) and set(self.scaling) == {"factor"}
+        if self.linear_scaling:
+            if not float(self.scaling["factor"]) > 0:
+                raise ValueError(f"scaling of rotary frequencies: a positive factor, got {self.scaling!r}")
+        elif self.scaling:
             missing = [k for k in ("factor", "low", "high", "original") if k not in self.scaling]
             if missing or self.scaling["high"] == self.scaling["low"]:
                 raise ValueError(f"scaling of rotary frequencies: factor, low, high (other than low) and original; "
@@ -107,7 +112,9 @@ class RotaryPositions(PositionEncoding):
             import torch
             i = torch.arange(self.dims // 2, dtype=torch.float64)
             f = self.base ** (-2.0 * i / max(self.dims, 1))
-            if self.scaling:
+            if self.linear_scaling:
+                f = f / float(self.scaling["factor"])
+            elif self.scaling:
                 import math
                 c = self.scaling
                 turns = float(c["original"]) * f / (2.0 * math.pi)        # original / wavelength
