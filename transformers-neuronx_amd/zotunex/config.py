@@ -91,14 +91,14 @@ class ZotunexConfig(ModelConfig):
             if layer.get("type") not in MIXERS:
                 raise ConfigError(f"key '{where}.type' must be one of {MIXERS}, got {layer.get('type')!r}")
             m, at = layer.get("mixer"), where + ".mixer"
-            for key in ("heads", "dim", "vdim"):
+            for key in ("heads", "dim") + (("vdim",) if layer["type"] != "attention" else ()):
                 _need(m, key, int, at)
             _need(m, "scale", float, at)
             if layer["type"] == "attention":
                 groups = _need(m, "kv_heads", int, at) if "kv_heads" in m else m["heads"]
                 if m["heads"] % groups:
                     raise ConfigError(f"key '{at}.heads' ({m['heads']}) must be a multiple of kv_heads ({groups})")
-                if m["vdim"] != m["dim"]:
+                if m.get("vdim", m["dim"]) != m["dim"]:
                     raise ConfigError(f"key '{at}.vdim' ({m['vdim']}) must equal dim ({m['dim']}): the values are the keys")
                 if m.get("rot") is not None:
                     _rotation(m["rot"], at + ".rot", m["dim"])

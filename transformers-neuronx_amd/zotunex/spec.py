@@ -18,6 +18,7 @@ def _rotary(rot, interleaved: bool) -> PartSpec:
 def zotunex_spec(cfg: ZotunexConfig) -> ModelSpec:
     d = cfg.width
     norm = PartSpec("rms_norm", dict(width=d, eps=cfg.eps, weight_suffix="", scalar=True))
+    no_norm = PartSpec("layer_norm", dict(width=d, eps=cfg.eps, affine=False))       # before a feed-forward that is not there
     layers, unread = [], []
     for i, layer in enumerate(cfg.layers):
         m = layer["mixer"]
@@ -49,7 +50,7 @@ def zotunex_spec(cfg: ZotunexConfig) -> ModelSpec:
                 router_name="router", correction_name="correction", route_scale=mlp["router"].get("scale", 1.0),
                 expert_name="e{}.", shared_name="shared.", names=("gate", "up", "down")))
         layers.append(LayerSpec(prefix=f"l{i}.", block="pre_norm", mixer=mixer, feed_forward=ffn, mixer_norm=norm,
-                                feed_forward_norm=norm, mixer_name="mix.", feed_forward_name="mlp.",
+                                feed_forward_norm=norm if mlp is not None else no_norm, mixer_name="mix.", feed_forward_name="mlp.",
                                 mixer_norm_name="norm1", feed_forward_norm_name="norm2"))
     embedding = PartSpec("token_table", dict(vocab=cfg.vocab, embed_width=d, width=d, position=PartSpec("none", {}),
                                              table_name="embed", projection_name=None, position_name=None,
