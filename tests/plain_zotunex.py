@@ -93,6 +93,24 @@ def causal_weights(scores, sink=None):
     return out
 
 
+def weights_over(scores, seen, sink=None):
+    """The same for queries that are a part of their sequence: scores `[H, I, J]`, `seen` `[I, J]` true where query
+    i may see key j."""
+    out = torch.zeros_like(scores)
+    for i in range(scores.shape[1]):
+        js = torch.nonzero(seen[i])[:, 0]
+        s = scores[:, i, js]
+        top = s.max(dim=-1, keepdim=True).values
+        if sink is not None:
+            top = torch.maximum(top, sink[:, None])
+        e = torch.exp(s - top)
+        denom = e.sum(-1, keepdim=True)
+        if sink is not None:
+            denom = denom + torch.exp(sink[:, None] - top)
+        out[:, i, js] = e / denom
+    return out
+
+
 # ---------------------------------------------------------------- the two mixers
 
 def attention(m, w, p, h, eps):
