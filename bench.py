@@ -93,6 +93,26 @@ def tadolix_config(width, heads, head, ff, vocab, layers, chunk=1024):
                         dict(type="parallel", mixer=pair, mlp=mlp) for i in range(layers)])
 
 
+def zotunex_config(width, heads, head, ff, vocab, layers):
+    """config.json contents of a Zotunex model at the sizes of a published layer: the first and every fourth layer
+    after it latent attention (heads of `head` + `head` / 2 query/key and `head` value elements over a latent of four
+    times `head`), the others attention whose values are its keys with a quarter as many key/value heads as query
+    heads and half of every head turned; the feed-forward by turns dense of `ff` and eight clamped experts of ff / 4
+    of which a token takes two, beside a shared one of ff / 2."""
+    attention = dict(heads=heads, kv_heads=max(1, heads // 4), dim=head, vdim=head, scale=head ** -0.5,
+                     rot=dict(base=500000.0, dims=head // 2, scaling=dict(factor=4.0)))
+    latent = dict(heads=heads, dim=head, rot_dim=head // 2, vdim=head, kv_rank=4 * head, scale=(head + head // 2) ** -0.5,
+                  rot=dict(base=10000.0, dims=head // 2))
+    dense = dict(kind="dense", ff=ff)
+    moe = dict(kind="moe", router=dict(experts=8, top=2, scale=1.5), expert=dict(ff=ff // 4, limit=7.0),
+               shared=dict(ff=ff // 2, limit=7.0))
+    return dict(architecture="Zotunex", vocab=vocab, width=width, norm=dict(eps=1e-6), embedding=dict(scale=width ** 0.5),
+                init_std=0.02, max_positions=4096,
+                layers=[dict(type="latent_attention" if i % 4 in (0, 3) else "attention",
+                             mixer=latent if i % 4 in (0, 3) else attention, mlp=moe if i % 2 else dense)
+                        for i in range(layers)])
+
+
 # a new design beside the closest one the engine had, at equal sizes: {design: {size: (its config, the other's)}};
 # the other's is the name of an OPT preset, or (design, its config)
 BESIDE = {"ratesun": {
@@ -105,6 +125,11 @@ BESIDE = {"ratesun": {
     "2048 wide": (lambda n: tadolix_config(2048, 32, 64, 8192, 50272, n),
                   ("sunatar", lambda n: sunatar_config(2048, 32, 64, 8192, 50272, n))),
     "4096 wide": (lambda n: tadolix_config(4096, 32, 128, 16384, 50272, n),
+                  ("sunatar", lambda n: sunatar_config(4096, 32, 128, 16384, 50272, n))),
+}, "zotunex": {
+    "2048 wide": (lambda n: zotunex_config(2048, 32, 64, 8192, 50272, n),
+                  ("sunatar", lambda n: sunatar_config(2048, 32, 64, 8192, 50272, n))),
+    "4096 wide": (lambda n: zotunex_config(4096, 32, 128, 16384, 50272, n),
                   ("sunatar", lambda n: sunatar_config(4096, 32, 128, 16384, 50272, n))),
 }}
 PREFILL_TOKENS = 2048

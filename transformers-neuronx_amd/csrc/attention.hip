@@ -566,7 +566,10 @@ __device__ __forceinline__ float tanh_by_exp(float x) {
   return 1.f - 2.f * __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(x * (2.f * LOG2E)));
 }
 
-template <int NDB, bool FAST, int GROUPS, bool SCORED = false>
+// MODS: 0, the plain kernel; 1, everything `ScoreMods` names; 2, what it names of the result alone (the gate, the
+// factor, rows that lie apart), the scores and the mask being the plain ones: the tiles' loop is then the plain
+// kernel's, with its registers.
+template <int NDB, bool FAST, int GROUPS, int MODS = 0>
 __global__ void __launch_bounds__(256 * GROUPS, (NDB <= 8 && GROUPS == 1 ? 2 : 1))
 attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                              const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
@@ -574,6 +577,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
                              int page_shift, int num_pages, const int* __restrict__ tile_run,
                              const int* __restrict__ tile_q0, bf16_t* __restrict__ out, int num_heads, int num_kv,
                              int head_size, int window, int page_pad, ScoreMods sm) {
+  constexpr bool SCORED = MODS == 1, RESULT = MODS != 0;
   constexpr int NKS = (NDB + 1) / 2;
   constexpr int DMAX = 16 * NDB;
   using Layout = PrefillTileLayout<NDB, FAST>;
@@ -945,7 +949,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   for (int qb = 0; qb < 2; ++qb) {
     const int qi = qw0 + 16 * qb + r;
     if (qi >= qlen) continue;
-    if (SCORED) {
+    if (RESULT) {
       const float inv = sm.out_scale / l[qb];
       bf16_t* orow = out + (size_t)(t0 + qi) * sm.out_ld + h * head_size;
       const float* gate = sm.gate ? sm.gate + (size_t)(t0 + qi) * sm.gate_ld + (size_t)h * sm.gate_head : nullptr;
@@ -983,7 +987,7 @@ attention_prefill_lds_kernel(const bf16_t* __restrict__ q, const bf16_t* __restr
   }
 }
 
-template <int NDB, bool FAST, int GROUPS, bool SCORED = false>
+template <int NDB, bool FAST, int GROUPS, int MODS = 0>
 static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
                               const bf16_t* v_pages, const int* run_start, const int* cached_lens, const int* table,
                               int table_width, int page_shift, int num_pages, const int* tile_run,
@@ -994,6 +998,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
   constexpr size_t tiles = GROUPS * 2 * (size_t)(Layout::KBUF + Layout::VBUF) * sizeof(bf16_t);
   constexpr size_t limit = 160 * 1024;
   size_t bytes = tiles;
+  constexpr bool SCORED = MODS == 1;
   if (SCORED) {
     // the head's bias row lies behind the tiles where LDS has the room
     const size_t row = sm.bias ? (size_t)(sm.far + 1) * sizeof(float) : 0;
@@ -1006,7 +1011,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
   static bool configured = false;
   if (!configured) {
     const size_t most = SCORED ? limit : tiles;
-    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST, GROUPS, SCORED>,
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_lds_kernel<NDB, FAST, GROUPS, MODS>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)most);
     if (e != hipSuccess) {
       tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", most, hipGetErrorString(e));
@@ -1014,7 +1019,7 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
     }
     configured = true;
   }
-  attention_prefill_lds_kernel<NDB, FAST, GROUPS, SCORED><<<grid, 256 * GROUPS, bytes, stream>>>(
+  attention_prefill_lds_kernel<NDB, FAST, GROUPS, MODS><<<grid, 256 * GROUPS, bytes, stream>>>(
       q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run, tile_q0, out,
       num_heads, num_kv, head_size, window, page_pad, sm);
   return 0;
@@ -1653,15 +1658,22 @@ extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, 
   grid, stream, (const bf16_t*)q, (const bf16_t*)k_pages, (const bf16_t*)v_pages, run_start, cached_lens, table, \
       table_width, page_shift, num_pages, tile_run, tile_q0, (bf16_t*)out, num_heads, num_kv, head_size, window, \
       page_pad, sm
-#define LAUNCH_SCORED(NDB)                                                                                           \
+#define LAUNCH_MODS(NDB, MODS)                                                                                       \
   {                                                                                                                  \
     constexpr int G = NDB <= 8 ? 2 : 1;                                                                              \
     const bool fast = NDB <= 8 && page_size >= 64 && head_size == 16 * NDB;                                          \
     if (sets == 1)                                                                                                   \
-      rc = fast ? launch_prefill_lds<NDB, true, 1, true>(SCORED_ARGS) : launch_prefill_lds<NDB, false, 1, true>(SCORED_ARGS); \
+      rc = fast ? launch_prefill_lds<NDB, true, 1, MODS>(SCORED_ARGS) : launch_prefill_lds<NDB, false, 1, MODS>(SCORED_ARGS); \
     else                                                                                                             \
-      rc = fast ? launch_prefill_lds<NDB, true, G, true>(SCORED_ARGS) : launch_prefill_lds<NDB, false, G, true>(SCORED_ARGS); \
+      rc = fast ? launch_prefill_lds<NDB, true, G, MODS>(SCORED_ARGS) : launch_prefill_lds<NDB, false, G, MODS>(SCORED_ARGS); \
   }
+  // plain scores under the plain mask: the result's part alone
+  const bool result_only = softcap == 0.f && bias == nullptr && chunk == 0;
+#define LAUNCH_SCORED(NDB)       \
+  if (result_only)               \
+    LAUNCH_MODS(NDB, 2)          \
+  else                           \
+    LAUNCH_MODS(NDB, 1)
   if (head_size <= 64) {
     LAUNCH_SCORED(4);
   } else if (head_size <= 128) {
@@ -1670,6 +1682,7 @@ extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, 
     LAUNCH_SCORED(16);
   }
 #undef LAUNCH_SCORED
+#undef LAUNCH_MODS
 #undef SCORED_ARGS
   if (rc) return rc;
   TNX_CHECK_LAUNCH("attention_prefill_scored");
