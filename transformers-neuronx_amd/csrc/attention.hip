@@ -1045,14 +1045,16 @@ static int launch_prefill_lds(dim3 grid, hipStream_t stream, const bf16_t* q, co
 // against 64.3 for the kernel above (per 64-key step of a block: 0.97 us is what the 136 matrix instructions of
 // its two waves a SIMD take, 1.8 us is what the step takes; LDS reads and the tile loads account for most of
 // the rest).
-template <int NDB, int GROUPS>
+// RESULT: what `ScoreMods` names of the result (the gate, the factor, rows that lie apart) is applied where the
+// result is written; scores and mask are the plain ones.
+template <int NDB, int GROUPS, bool RESULT = false>
 __global__ void __launch_bounds__(256 * GROUPS, GROUPS == 1 ? 2 : 1)
 attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k_pages,
                                    const bf16_t* __restrict__ v_pages, const int* __restrict__ run_start,
                                    const int* __restrict__ cached_lens, const int* __restrict__ table,
                                    int table_width, int page_shift, int num_pages,
                                    const int* __restrict__ tile_run, const int* __restrict__ tile_q0,
-                                   bf16_t* __restrict__ out, int num_heads, int num_kv, int page_pad) {
+                                   bf16_t* __restrict__ out, int num_heads, int num_kv, int page_pad, ScoreMods sm) {
   static_assert(NDB == 4 || NDB == 8, "head sizes 64 and 128");
   constexpr int NKS = NDB / 2, DH = 16 * NDB, CPR = 2 * NDB;   // CPR: 16-byte chunks of a key row
   constexpr int TILE_BYTES = 64 * DH * 2;                       // 64 keys, and as many values
@@ -1507,6 +1509,29 @@ attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* _
   for (int qb = 0; qb < 2; ++qb) {
     const int qi = qw0 + 16 * qb + r;
     if (qi >= qlen) continue;
+    if (RESULT) {
+      const float inv = sm.out_scale / l[qb];
+      bf16_t* orow = out + (size_t)(t0 + qi) * sm.out_ld + h * DH;
+      const float* gate = sm.gate ? sm.gate + (size_t)(t0 + qi) * sm.gate_ld + (size_t)h * sm.gate_head : nullptr;
+#pragma unroll
+      for (int db = 0; db < NDB; ++db) {
+        const int d0 = 16 * db + 4 * g;
+        bf16x4 v4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          float x = o[db][qb][i] * inv;
+          if (gate) x *= __builtin_amdgcn_rcpf(1.f + __builtin_amdgcn_exp2f(-gate[sm.gate_head == 1 ? 0 : d0 + i] * LOG2E));
+          v4[i] = (bf16_t)x;
+        }
+        if (sm.vector_store) {
+          *(bf16x4*)(orow + d0) = v4;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) orow[d0 + i] = v4[i];
+        }
+      }
+      continue;
+    }
     const float inv = 1.f / l[qb];
     bf16_t* orow = out + (size_t)(t0 + qi) * nq + h * DH;
 #pragma unroll
@@ -1519,19 +1544,19 @@ attention_prefill_pipelined_kernel(const bf16_t* __restrict__ q, const bf16_t* _
   }
 }
 
-template <int NDB, int GROUPS>
+template <int NDB, int GROUPS, bool RESULT = false>
 static int launch_prefill_pipelined(dim3 grid, hipStream_t stream, const bf16_t* q, const bf16_t* k_pages,
                                     const bf16_t* v_pages, const int* run_start, const int* cached_lens,
                                     const int* table, int table_width, int page_shift, int num_pages,
                                     const int* tile_run, const int* tile_q0, bf16_t* out, int num_heads, int num_kv,
-                                    int head_size, int window, int page_pad) {
+                                    int head_size, int window, int page_pad, ScoreMods sm = ScoreMods{}) {
   constexpr size_t bytes = GROUPS * 4 * (size_t)(64 * 16 * NDB * 2);
   static_assert(bytes <= 160 * 1024, "the staging buffers must fit the 160 KB of LDS");
   static_assert(GROUPS == 1 || bytes >= (4 * NDB * 2 * 4 * 64 + 4 * 2 * 2 * 64) * sizeof(float),
                 "the partial results of the second set of waves must fit the staging buffers");
   static bool configured = false;
   if (!configured) {
-    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_pipelined_kernel<NDB, GROUPS>,
+    hipError_t e = hipFuncSetAttribute((const void*)attention_prefill_pipelined_kernel<NDB, GROUPS, RESULT>,
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
     if (e != hipSuccess) {
       tnx_set_error("attention_prefill: cannot reserve %zu bytes of LDS: %s", bytes, hipGetErrorString(e));
@@ -1541,9 +1566,9 @@ static int launch_prefill_pipelined(dim3 grid, hipStream_t stream, const bf16_t*
   }
   (void)head_size;
   (void)window;
-  attention_prefill_pipelined_kernel<NDB, GROUPS><<<grid, 256 * GROUPS, bytes, stream>>>(
+  attention_prefill_pipelined_kernel<NDB, GROUPS, RESULT><<<grid, 256 * GROUPS, bytes, stream>>>(
       q, k_pages, v_pages, run_start, cached_lens, table, table_width, page_shift, num_pages, tile_run, tile_q0, out,
-      num_heads, num_kv, page_pad);
+      num_heads, num_kv, page_pad, sm);
   return 0;
 }
 
@@ -1674,7 +1699,13 @@ extern "C" int tnx_attention_prefill_scored(const void* q, const void* k_pages, 
     LAUNCH_MODS(NDB, 2)          \
   else                           \
     LAUNCH_MODS(NDB, 1)
-  if (head_size <= 64) {
+  if (result_only && window <= 0 && page_size >= 64 && value_size == head_size && (head_size == 64 || head_size == 128)) {
+    // the pipelined kernel takes these, as it does for the plain call
+    if (head_size == 64)
+      rc = sets == 2 ? launch_prefill_pipelined<4, 2, true>(SCORED_ARGS) : launch_prefill_pipelined<4, 1, true>(SCORED_ARGS);
+    else
+      rc = sets == 2 ? launch_prefill_pipelined<8, 2, true>(SCORED_ARGS) : launch_prefill_pipelined<8, 1, true>(SCORED_ARGS);
+  } else if (head_size <= 64) {
     LAUNCH_SCORED(4);
   } else if (head_size <= 128) {
     LAUNCH_SCORED(8);
