@@ -77,7 +77,7 @@ def rotate_halves(x, positions, rot):
 
 def causal_weights(scores, sink=None):
     """scores `[H, T, T]` (query i, key j): the softmax over j <= i, query by query. `sink` `[H]`: the denominator
-    also holds exp(sink) of the head, once, with no key and no value behind it."""
+    also holds exp(sink) of the head, once: a term that stands for no token and adds nothing to the sum of values."""
     heads, t, _ = scores.shape
     out = torch.zeros_like(scores)
     for i in range(t):

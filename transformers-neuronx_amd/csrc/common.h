@@ -173,7 +173,7 @@ __device__ __forceinline__ float apply_act(float x, int act) {
 
 // What a softmax's running maximum `m` and sum `l` (of exp(score - m) over the visible keys) make of the weighted
 // sum that was gathered with them: the factor 1 / l. With a sink (`sink` non-null: the head's number) the
-// denominator holds exp(sink) once more, with no key and no value behind it; with a gate (`gate` non-null: the
+// denominator holds exp(sink) once more, a term that stands for no token; with a gate (`gate` non-null: the
 // (token, head)'s number) the result is multiplied by sigmoid(gate). Full-precision exponentials: once a row.
 __device__ __forceinline__ float softmax_finish(float m, float l, const float* sink, const float* gate) {
   float f;

@@ -345,8 +345,8 @@ class LatentAttention(Mixer):
     the step, and a (query, key) pair costs 2 (n + r + v) multiply-adds a head instead of 2 (2R + r).
 
     `q_rank=None`: no query latent: q = W_q h, one matrix (the second of `names`; the first is not read).
-    `sink`: the name of a tensor of one number a head; the softmax's denominator also holds exp(sink), once, with no
-    key and no value behind it. `out_gate`: the name of a matrix W_g `[heads, width]`; a head's result is multiplied
+    `sink`: the name of a tensor of one number a head; the softmax's denominator also holds exp(sink), once, a term
+    that stands for no token. `out_gate`: the name of a matrix W_g `[heads, width]`; a head's result is multiplied
     by sigmoid(W_g h) of that head before W_o (its rows ride in the product with W_dkv). A rotation that pairs
     element i with i + dims / 2 is brought to neighbouring pairs by putting the rows of the matrices that make
     q_r and k_r in the order (0, dims/2, 1, dims/2 + 1, ...) once, at load: q_r and k_r meet in a dot product
