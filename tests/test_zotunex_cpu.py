@@ -240,7 +240,7 @@ def test_the_stream_after_every_layer():
     with debug.debug_context() as taps:
         runner.step([StepEntry("r0", toks, [])])
     for i, want in enumerate(layers):
-        got = taps.tensors[f"call{i}.layer{i}"] if hasattr(taps, "tensors") else taps[f"call{i}.layer{i}"]
+        got = taps[f"call{i}.layer{i}"]
         assert float((got.double() - want).abs().max() / want.abs().max()) < 1e-5, i
 
 

@@ -390,7 +390,7 @@ def test_the_stream_after_every_layer_on_the_gpu():
     with debug.debug_context() as taps:
         runner.step([StepEntry("r0", toks, [])])
     for i, want in enumerate(layers):
-        got = taps.tensors[f"call{i}.layer{i}"] if hasattr(taps, "tensors") else taps[f"call{i}.layer{i}"]
+        got = taps[f"call{i}.layer{i}"]
         assert float((got.double().cpu() - want).abs().max() / want.abs().max()) < 1e-5, i
 
 
